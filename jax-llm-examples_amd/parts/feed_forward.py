@@ -1,0 +1,75 @@
+"""Feed-forward parts.
+
+``dense_swiglu``: ``(silu(x Wg) * (x Wu)) Wd`` (``llama4/llama4_jax/model.py:1142-1153``).
+``moe_sigmoid_shared``: router logits in float32, the ``top_k`` largest per token,
+gate = sigmoid of the chosen logit, the gate multiplies the expert's *input*
+(``model.py:958-972, 1066-1071``), SwiGLU experts (``model.py:1076-1085``), sum
+over the chosen experts (``model.py:1111``), plus one shared SwiGLU expert on the
+unscaled input (``model.py:1137-1139``).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .base import FeedForward, ParamSpec, register_feed_forward
+
+
+@register_feed_forward("dense_swiglu")
+class DenseSwiGLU(FeedForward):
+    def __init__(self, spec) -> None:
+        super().__init__()
+        self.hidden = int(spec.hidden_size)
+        self.inter = int(spec.intermediate_size)
+
+    def param_specs(self):
+        return {
+            "w_gate_up": ParamSpec((2 * self.inter, self.hidden)),  # gate rows, then up rows
+            "w_down": ParamSpec((self.hidden, self.inter)),
+        }
+
+    def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
+        ops = ctx.ops
+        act = ops.silu_mul(ops.linear(h, self.params["w_gate_up"]))
+        return ops.linear(act, self.params["w_down"])
+
+
+@register_feed_forward("moe_sigmoid_shared")
+class MoESigmoidShared(FeedForward):
+    wants_float32_input = True
+
+    def __init__(self, spec) -> None:
+        super().__init__()
+        self.hidden = int(spec.hidden_size)
+        self.num_experts = int(spec.num_experts)
+        self.top_k = int(spec.top_k)
+        self.inter = int(spec.intermediate_size)
+        self.shared_inter = int(spec.get("shared_intermediate_size") or 0)
+        self.last_routing = None  # (expert ids, gates) of the latest call, for tests
+
+    def param_specs(self):
+        e, f, d = self.num_experts, self.inter, self.hidden
+        specs = {
+            "router": ParamSpec((e, d), policy="float32"),
+            "w_gate_up": ParamSpec((e, 2 * f, d)),  # per expert [out, in]: gate rows, then up rows
+            "w_down": ParamSpec((e, d, f)),
+        }
+        if self.shared_inter:
+            specs["shared_gate_up"] = ParamSpec((2 * self.shared_inter, d))
+            specs["shared_down"] = ParamSpec((d, self.shared_inter))
+        return specs
+
+    def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
+        ops = ctx.ops
+        expert_ids, gates = ops.moe_route(h32, self.params["router"], self.top_k)
+        if ctx.record_routing:
+            self.last_routing = (expert_ids.clone(), gates.clone())
+        forced = ctx.forced_routing.get(id(self)) if ctx.forced_routing else None
+        if forced is not None:
+            expert_ids, gates = forced
+        shared = None
+        if self.shared_inter:
+            act = ops.silu_mul(ops.linear(h, self.params["shared_gate_up"]))
+            shared = ops.linear(act, self.params["shared_down"])
+        return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"], shared)

@@ -1,0 +1,41 @@
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.dirname(os.path.abspath(__file__))):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an AMD GPU (run on the MI355X box)")
+
+
+def pytest_collection_modifyitems(config, items):
+    if torch.cuda.is_available():
+        return
+    skip = pytest.mark.skip(reason="no GPU in this machine")
+    for item in items:
+        if "gpu" in item.keywords:
+            item.add_marker(skip)
+
+
+@pytest.fixture(scope="session")
+def model_dirs(tmp_path_factory):
+    """Model folders (config.json + model.safetensors) of the tiny configurations,
+    written once per session into a temporary folder, in float32."""
+    from tiny_configs import TINY, write_tiny
+
+    root = tmp_path_factory.mktemp("models")
+    return {name: write_tiny(name, str(root / name), torch.float32) for name in TINY}
+
+
+@pytest.fixture(scope="session")
+def model_dirs_bf16(tmp_path_factory):
+    from tiny_configs import TINY, write_tiny
+
+    root = tmp_path_factory.mktemp("models_bf16")
+    return {name: write_tiny(name, str(root / name), torch.bfloat16) for name in TINY}

@@ -1,0 +1,57 @@
+"""Two tiny Llama 4 configurations that differ in every size and option."""
+import torch
+
+TINY = {
+    # all layers with experts, qk norm, temperature tuning, no frequency scaling, layer 3 NoPE
+    "A": {
+        "architectures": ["Llama4ForCausalLM"],
+        "seed": 11,
+        "num_hidden_layers": 4, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2,
+        "head_dim": 16, "interleave_moe_layer_step": 1, "num_local_experts": 4, "num_experts_per_tok": 1,
+        "intermediate_size": 128, "intermediate_size_mlp": 256, "vocab_size": 512, "rope_theta": 10000.0,
+        "rope_scaling": None, "no_rope_layers": [1, 1, 1, 0], "attention_chunk_size": 32, "use_qk_norm": True,
+        "attn_temperature_tuning": True, "floor_scale": 16, "attn_scale": 0.1, "rms_norm_eps": 1e-5,
+        "tie_word_embeddings": False,
+    },
+    # experts on every 2nd layer, dense elsewhere, no qk norm, no temperature, llama3 scaling, multimodal naming
+    "B": {
+        "architectures": ["Llama4ForConditionalGeneration"],
+        "seed": 23,
+        "text_config": {
+            "num_hidden_layers": 6, "hidden_size": 96, "num_attention_heads": 6, "num_key_value_heads": 3,
+            "head_dim": 32, "interleave_moe_layer_step": 2, "num_local_experts": 8, "num_experts_per_tok": 1,
+            "intermediate_size": 64, "intermediate_size_mlp": 192, "vocab_size": 1000, "rope_theta": 500000.0,
+            "rope_scaling": {"rope_type": "llama3", "factor": 4.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                             "original_max_position_embeddings": 64},
+            "no_rope_layers": [1, 1, 0, 1, 1, 0], "attention_chunk_size": 48, "use_qk_norm": False,
+            "attn_temperature_tuning": False, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+        },
+    },
+    # odd sizes: width and vocabulary that are no power of two, 5 heads in one group, head size 48,
+    # two experts per token, a chunk that is no multiple of the page size
+    "C": {
+        "architectures": ["Llama4ForCausalLM"],
+        "seed": 37,
+        "num_hidden_layers": 3, "hidden_size": 80, "num_attention_heads": 5, "num_key_value_heads": 1,
+        "head_dim": 48, "interleave_moe_layer_step": 1, "moe_layers": [0, 2], "num_local_experts": 3,
+        "num_experts_per_tok": 2, "intermediate_size": 40, "intermediate_size_mlp": 56, "vocab_size": 311,
+        "rope_theta": 1000.0, "rope_scaling": None, "no_rope_layers": [1, 0, 1], "attention_chunk_size": 20,
+        "use_qk_norm": True, "attn_temperature_tuning": True, "floor_scale": 7, "attn_scale": 0.25,
+        "rms_norm_eps": 1e-4, "tie_word_embeddings": False,
+    },
+}
+
+
+def tiny_config_json(name: str) -> dict:
+    c = {k: v for k, v in TINY[name].items() if k != "seed"}
+    return c
+
+
+def write_tiny(name: str, out_dir: str, dtype=torch.float32) -> str:
+    from jax_llm_examples_amd.config import get_architecture
+    from jax_llm_examples_amd.weights import write_random_model
+
+    top = tiny_config_json(name)
+    arch = get_architecture(top["architectures"][0])
+    cfg = arch.parse_config(top)
+    return write_random_model(arch, cfg, out_dir, TINY[name]["seed"], dtype, architecture=top["architectures"][0])
