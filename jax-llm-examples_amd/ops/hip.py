@@ -1,0 +1,264 @@
+"""The engine's kernel set on the GPU: hand-written HIP kernels (``csrc/``) called
+through a C interface, plus library matrix products for the dense projections
+(where the reference uses its library's ``einsum``, ``llama4/llama4_jax/model.py:907-909,
+952-954, 1146-1152, 1204``).  Kernels run on PyTorch's current stream.  There is no
+fallback: if the library cannot be built or loaded, constructing :class:`HipOps` fails.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build as _build
+
+_RET_MODES = {"all": 0, "chunk": 1, "window": 2}
+
+_vp, _i, _f, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_longlong
+
+_SIGNATURES = {
+    "jle_embed": [_vp, _vp, _i, _vp, _i, _i, _vp],
+    "jle_add_rmsnorm": [_vp, _vp, _i, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
+    "jle_add_residual": [_vp, _vp, _i, _ll, _vp],
+    "jle_gather_rows": [_vp, _vp, _vp, _i, _i, _vp],
+    "jle_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
+    "jle_moe_combine": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "jle_qk_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_paged_attention_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_moe_route": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_LIB = None
+
+
+def load_library():
+    """Loads the compiled kernels (compiling them if no build is there)."""
+    global _LIB
+    if _LIB is None:
+        path = _build.library_path()
+        try:
+            lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError(f"cannot load the HIP kernel library {path}: {e}") from e
+        for name, args in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = ctypes.c_int
+        lib._jle_path = path
+        _LIB = lib
+    return _LIB
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+class HipOps:
+    name = "hip"
+
+    def __init__(self, device) -> None:
+        self.device = torch.device(device)
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise KernelError("the HIP kernels need a GPU")
+        self.lib = load_library()
+        # true float32 products: no reduced-precision matrix mode
+        torch.backends.cuda.matmul.allow_tf32 = False
+        torch.backends.cudnn.allow_tf32 = False
+        torch.set_float32_matmul_precision("highest")
+
+    # ------------------------------------------------------------------ helpers
+    def _stream(self):
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _call(self, name: str, *args) -> None:
+        rc = getattr(self.lib, name)(*args, self._stream())
+        if rc != 0:
+            if rc < 0:
+                raise KernelError(f"{name}: the kernel refuses these sizes or options")
+            raise KernelError(f"{name}: HIP error {rc}")
+
+    @staticmethod
+    def _is_bf16(t: torch.Tensor) -> int:
+        if t.dtype == torch.bfloat16:
+            return 1
+        if t.dtype == torch.float32:
+            return 0
+        raise KernelError(f"unsupported dtype {t.dtype}")
+
+    @staticmethod
+    def _chk(t: torch.Tensor, dtype=None, shape=None, what: str = "tensor") -> torch.Tensor:
+        if not t.is_cuda:
+            raise KernelError(f"{what} must be on the GPU")
+        if not t.is_contiguous():
+            raise KernelError(f"{what} must be contiguous, got strides {t.stride()} for shape {tuple(t.shape)}")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{what} must be {dtype}, got {t.dtype}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{what} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+        return t
+
+    # ------------------------------------------------------------------ embedding, norms
+    def embed(self, token_ids, table):
+        n, (v, d) = token_ids.numel(), table.shape
+        self._chk(token_ids, torch.int32, (n,), "token ids")
+        self._chk(table, None, (v, d), "embedding table")
+        out = torch.empty(n, d, dtype=torch.float32, device=table.device)
+        self._call("jle_embed", _p(token_ids), _p(table), self._is_bf16(table), _p(out), n, d)
+        return out
+
+    def add_rmsnorm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False):
+        n, d = x.shape
+        self._chk(x, torch.float32, (n, d), "residual")
+        if delta is not None:
+            self._chk(delta, None, (n, d), "branch output")
+        if weight is not None:
+            self._chk(weight, torch.float32, (d,), "norm weight")
+        out = torch.empty(n, d, dtype=out_dtype, device=x.device)
+        out32 = torch.empty(n, d, dtype=torch.float32, device=x.device) if want32 else None
+        self._call("jle_add_rmsnorm", _p(x), _p(delta), 0 if delta is None else self._is_bf16(delta), _p(weight),
+                   float(eps), _p(out), self._is_bf16(out), _p(out32), n, d)
+        return out, out32
+
+    def add_residual(self, x, delta) -> None:
+        self._chk(x, torch.float32, None, "residual")
+        self._chk(delta, None, x.shape, "branch output")
+        self._call("jle_add_residual", _p(x), _p(delta), self._is_bf16(delta), x.numel())
+
+    def gather_rows(self, x, idx):
+        m = idx.numel()
+        self._chk(x, None, None, "rows")
+        self._chk(idx, torch.int32, (m,), "row indices")
+        out = torch.empty(m, x.shape[1], dtype=x.dtype, device=x.device)
+        self._call("jle_gather_rows", _p(x), _p(idx), _p(out), m, x.shape[1] * x.element_size())
+        return out
+
+    # ------------------------------------------------------------------ matrix products
+    def linear(self, h, w, out_dtype=None):
+        """``h @ w.T`` through the BLAS library (float32: true float32)."""
+        out = torch.matmul(h, w.t())
+        return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
+
+    def gemm(self, a, b, *, offsets=None, a_rows=None, scale=None, out_f32=False, rows=None):
+        """The hand-written product ``C[r] = scale[r] * A[a_rows[r]] @ B[g(r)].T`` (see ``gemm_generic.hip``)."""
+        if b.dim() == 2:
+            b = b.unsqueeze(0)
+        g, nout, k = b.shape
+        m = rows if rows is not None else (a_rows.numel() if a_rows is not None else a.shape[0])
+        self._chk(a, b.dtype, None, "A")
+        self._chk(b, None, None, "B")
+        if a.shape[1] != k:
+            raise KernelError(f"inner sizes differ: A {tuple(a.shape)}, B {tuple(b.shape)}")
+        out = torch.empty(m, nout, dtype=torch.float32 if out_f32 else a.dtype, device=a.device)
+        self._call("jle_gemm_generic", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), self._is_bf16(a),
+                   1 if (out_f32 or a.dtype == torch.float32) else 0, m, nout, k, g)
+        return out
+
+    def lm_head(self, h, w):
+        if h.dtype == torch.float32:
+            return torch.matmul(h, w.t())
+        return self.gemm(h, w, out_f32=True)
+
+    def silu_mul(self, gate_up):
+        n, f2 = gate_up.shape
+        self._chk(gate_up, None, None, "gate|up")
+        out = torch.empty(n, f2 // 2, dtype=gate_up.dtype, device=gate_up.device)
+        self._call("jle_silu_mul", _p(gate_up), _p(out), self._is_bf16(gate_up), n, f2 // 2)
+        return out
+
+    # ------------------------------------------------------------------ attention
+    def qk_prepare_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, qk_norm_eps,
+                            query_scale, kv_cache, slot_mapping):
+        n = qkv.shape[0]
+        hq, hk, dh = num_heads, num_kv_heads, head_dim
+        self._chk(qkv, None, (n, (hq + 2 * hk) * dh), "q|k|v")
+        self._chk(positions, torch.int32, (n,), "positions")
+        if inv_freq is not None:
+            self._chk(inv_freq, torch.float32, (dh // 2,), "inv_freq")
+        ps = 0
+        if kv_cache is not None:
+            ps = kv_cache.shape[3]
+            self._chk(kv_cache, qkv.dtype, (kv_cache.shape[0], 2, hk, ps, dh), "kv pages")
+            self._chk(slot_mapping, torch.int32, (n,), "slot mapping")
+        q = torch.empty(n, hq, dh, dtype=qkv.dtype, device=qkv.device)
+        fs, sc = (query_scale if query_scale is not None else (0.0, 0.0))
+        self._call("jle_qk_prepare", _p(qkv), _p(q), _p(kv_cache), _p(positions),
+                   _p(slot_mapping) if kv_cache is not None else None, _p(inv_freq),
+                   -1.0 if qk_norm_eps is None else float(qk_norm_eps), float(fs), float(sc), self._is_bf16(qkv),
+                   n, hq, hk, dh, max(ps, 1), 0 if kv_cache is None else 1)
+        return q
+
+    def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
+        n, hq, dh = q.shape
+        hk, ps = kv_cache.shape[2], kv_cache.shape[3]
+        self._chk(q, kv_cache.dtype, None, "q")
+        self._chk(kv_cache, None, (kv_cache.shape[0], 2, hk, ps, dh), "kv pages")
+        self._chk(block_table, torch.int32, None, "block table")
+        self._chk(positions, torch.int32, (n,), "positions")
+        self._chk(token_segment, torch.int32, (n,), "token segments")
+        mode = _RET_MODES[retention[0]]
+        param = int(retention[1]) if len(retention) > 1 else 0
+        out = torch.empty(n, hq * dh, dtype=q.dtype, device=q.device)
+        self._call("jle_paged_attention_generic", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
+                   _p(block_table), block_table.shape[1], mode, param, float(scale), self._is_bf16(q), n, hq, hk, dh,
+                   ps)
+        return out
+
+    # ------------------------------------------------------------------ routed experts
+    def moe_route(self, h32, router, top_k: int, want_logits: bool = False):
+        n, d = h32.shape
+        e = router.shape[0]
+        self._chk(h32, torch.float32, None, "router input")
+        self._chk(router, torch.float32, (e, d), "router matrix")
+        ids = torch.empty(n, top_k, dtype=torch.int32, device=h32.device)
+        gates = torch.empty(n, top_k, dtype=torch.float32, device=h32.device)
+        logits = torch.empty(n, e, dtype=torch.float32, device=h32.device) if want_logits else None
+        self._call("jle_moe_route", _p(h32), _p(router), _p(ids), _p(gates), _p(logits), n, d, e, top_k)
+        return (ids, gates, logits) if want_logits else (ids, gates)
+
+    def moe_align(self, expert_ids, gates, num_experts: int):
+        n, k = expert_ids.shape
+        m = n * k
+        dev = expert_ids.device
+        self._chk(expert_ids, torch.int32, None, "expert ids")
+        self._chk(gates, torch.float32, (n, k), "gates")
+        offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
+        sorted_token = torch.empty(m, dtype=torch.int32, device=dev)
+        sorted_gate = torch.empty(m, dtype=torch.float32, device=dev)
+        inv = torch.empty(m, dtype=torch.int32, device=dev)
+        self._call("jle_moe_align", _p(expert_ids), _p(gates), _p(offsets), _p(sorted_token), _p(sorted_gate), _p(inv),
+                   m, num_experts, k)
+        return offsets, sorted_token, sorted_gate, inv
+
+    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None):
+        n, d = h.shape
+        e, f2, _ = w_gate_up.shape
+        k = expert_ids.shape[1]
+        offsets, sorted_token, sorted_gate, inv = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e)
+        gu = self.gemm(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate)
+        act = self.silu_mul(gu)
+        routed = self.gemm(act, w_down, offsets=offsets)
+        out = torch.empty(n, d, dtype=torch.float32, device=h.device)
+        if shared is not None:
+            self._chk(shared, h.dtype, (n, d), "shared expert output")
+        self._call("jle_moe_combine", _p(routed), _p(inv), _p(shared), _p(out), self._is_bf16(h), n, k, d)
+        return out
+
+    # ------------------------------------------------------------------ sampling
+    def sample(self, logits, temperature, top_k, seeds, counters):
+        m, v = logits.shape
+        self._chk(logits, torch.float32, None, "logits")
+        self._chk(temperature, torch.float32, (m,), "temperature")
+        for t, what in ((top_k, "top_k"), (seeds, "seeds"), (counters, "counters")):
+            self._chk(t, torch.int32, (m,), what)
+        out = torch.empty(m, dtype=torch.int32, device=logits.device)
+        self._call("jle_sample", _p(logits), _p(temperature), _p(top_k), _p(seeds), _p(counters), _p(out), m, v)
+        return out
