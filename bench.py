@@ -1,0 +1,177 @@
+"""Decode and prefill throughput of the Llama 4 Scout layer sizes with random weights on
+one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+prints one JSON line: ``value`` = decoded tokens per second at batch 8 and context 4,096
+(a "step" is one decode step of the whole batch, sampling included), plus the prefill of
+2,048 tokens, the decode step's HBM roofline fraction, and decode at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0  # MI355X: HBM3E 8 TB/s
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}  # dense MFMA
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration's 48")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
+    ap.add_argument("--point-steps", type=int, default=12)
+    ap.add_argument("--preset", default="llama4-scout")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this engine runs on one GPU; --gpus > 1 is not supported")
+        return 2
+
+    import torch
+
+    from jax_llm_examples_amd.cache import CacheManager
+    from jax_llm_examples_amd.config.presets import PRESETS, preset
+    from jax_llm_examples_amd.config.registry import architecture_name, get_architecture
+    from jax_llm_examples_amd.engine import ModelRunner, StepEntry, get_ops, random_model
+    from jax_llm_examples_amd.engine.accounting import decode_step_bytes, prefill_flops
+    from jax_llm_examples_amd.parts.feed_forward import MoESigmoidShared
+    from jax_llm_examples_amd.sampling import Sampler, SamplingParams
+
+    dev = "cuda:0"
+    full_layers = PRESETS[args.preset]["num_hidden_layers"]
+    layers = args.layers or full_layers
+    top = preset(args.preset, layers)
+    arch = get_architecture(architecture_name(top))
+    cfg = arch.parse_config(top)
+    t0 = time.time()
+    model = random_model(arch, cfg, seed=0, dtype=args.dtype, device=dev)
+    torch.cuda.synchronize()
+    print(f"[bench] {layers}-layer model with random weights on the GPU after {time.time() - t0:.0f} s "
+          f"({model.num_parameters() / 1e9:.1f} B parameters)", file=sys.stderr, flush=True)
+
+    page = 16
+    batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
+    need_tokens = max(batches) * (args.context + page) + args.prefill_tokens + 4 * page
+    ops = get_ops(dev)
+    cache = CacheManager(model.cache_needs(), page_size=page, num_pages=-(-need_tokens // page),
+                         max_requests=max(batches) + 1, dtype=model.dtype, device=dev)
+    for g in cache.groups:  # stand-in keys and values for contexts that are not computed
+        for t in g.tensors.values():
+            step = max(1, (1 << 28) // max(1, t[0].numel()))
+            for o in range(0, t.shape[0], step):
+                t[o: o + step].normal_(0.0, 0.5)
+    runner = ModelRunner(model, cache, ops)
+    sampler = Sampler(ops, dev)
+    gen = torch.Generator().manual_seed(0)
+    V = model.plan.vocab_size
+    greedy = SamplingParams()
+    dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
+
+    # ------------------------------------------------------------------ prefill of 2,048 tokens
+    prefill = None
+    if not args.no_prefill:
+        T = args.prefill_tokens
+        times = []
+        for it in range(3):
+            toks = torch.randint(0, V, (T,), generator=gen).tolist()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            logits = runner.step([StepEntry(f"p{it}", toks, [T - 1])])
+            sampler(logits, [greedy], [0])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t1)
+            runner.finish(f"p{it}")
+            print(f"[bench] prefill of {T} tokens: {times[-1] * 1e3:.1f} ms", file=sys.stderr, flush=True)
+        sec = min(times[1:])
+        fl = prefill_flops(model, T)
+        prefill = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 2),
+                   "frac": round(fl / sec / PEAK_FLOPS[dkey], 4)}
+
+    # ------------------------------------------------------------------ decode
+    def decode(batch: int, steps: int, warmup: int):
+        ctx0 = args.context - (steps + warmup)
+        ids = [f"d{batch}_{i}" for i in range(batch)]
+        for rid in ids:  # contexts stand in: pages are taken, their contents are the random fill
+            cache.add_request(rid)
+            cache.reserve(rid, ctx0)
+            cache.commit(rid)
+        last = torch.randint(0, V, (batch,), generator=gen).tolist()
+        params, ctr = [greedy] * batch, [0] * batch
+
+        def one(record=False):
+            nonlocal last
+            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(ids, last)], record_routing=record)
+            last = sampler(logits, params, ctr)
+
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t1) / steps
+        distinct = {}
+        one(record=True)
+        for li, b in enumerate(model.blocks):
+            ff = b.feed_forward
+            if isinstance(ff, MoESigmoidShared) and ff.last_routing is not None:
+                distinct[li] = int(torch.unique(ff.last_routing[0]).numel())
+        contexts = [cache.num_tokens(r) for r in ids]
+        nbytes = decode_step_bytes(model, cache, contexts, distinct)
+        for rid in ids:
+            runner.finish(rid)
+        print(f"[bench] decode batch {batch}: {sec * 1e3:.2f} ms/step, {batch / sec:.1f} tok/s, "
+              f"{nbytes['total'] / 1e9:.1f} GB/step -> {nbytes['total'] / sec / 1e9:.0f} GB/s", file=sys.stderr,
+              flush=True)
+        return sec, nbytes, (sum(distinct.values()) / max(1, len(distinct)))
+
+    sec, nbytes, mean_experts = decode(args.batch, args.steps, args.warmup)
+    points = {}
+    for b in batches[1:]:
+        s, _, _ = decode(b, args.point_steps, 2)
+        points[f"decode_b{b}"] = round(b / s, 1)
+
+    achieved = nbytes["total"] / sec / 1e9
+    out = {
+        "metric": "decode tok/s at batch 8, context 4096 (Llama 4 Scout layer sizes, random weights)",
+        "value": round(args.batch / sec, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dkey,
+        "data": "synthetic: random token ids, seeded random weights, decode contexts filled with random keys/values",
+        "config": {
+            "model": args.preset, "num_layers": layers, "num_layers_full": full_layers,
+            "hidden_size": cfg.hidden_size, "num_heads": cfg.num_attention_heads,
+            "num_kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "num_experts": cfg.num_local_experts,
+            "experts_per_tok": cfg.num_experts_per_tok, "expert_intermediate": cfg.intermediate_size,
+            "mlp_intermediate": cfg.intermediate_size_mlp, "vocab_size": cfg.vocab_size,
+            "attention_chunk": cfg.attention_chunk_size, "global_batch": args.batch, "seq_len": args.context,
+            "prefill_tokens": args.prefill_tokens, "page_size": page, "parallelism": "single-gpu",
+            "mean_distinct_experts": round(mean_experts, 2),
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
