@@ -20,6 +20,7 @@ class PagePool:
         self.num_pages = num_pages
         self._free = list(range(num_pages - 1, -1, -1))
         self._held = bytearray(num_pages)
+        self.handed_out = 0  # pages given out so far (more than num_pages: pages were used again)
 
     @property
     def num_free(self) -> int:
@@ -33,6 +34,7 @@ class PagePool:
         if n > len(self._free):
             raise OutOfPages(f"asked for {n} pages, {len(self._free)} of {self.num_pages} free")
         out = [self._free.pop() for _ in range(n)]
+        self.handed_out += n
         for p in out:
             if self._held[p]:
                 raise AssertionError(f"page {p} handed out twice")

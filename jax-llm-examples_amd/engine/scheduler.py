@@ -144,6 +144,13 @@ class Scheduler:
             planned.add(id(r))
             return True
 
+        def recount() -> None:
+            """Free pages after a request gave back what it held, less what this step's segments will take."""
+            free[:] = self.cache.num_free_pages()
+            for s in segments:
+                for g, x in enumerate(self._needed(s.request, s.count)):
+                    free[g] -= x
+
         # 1. running requests, decoding ones first, each in order of admission
         order = [r for r in self.running if r.num_pending == 1] + [r for r in self.running if r.num_pending != 1]
         for r in order:
@@ -157,13 +164,11 @@ class Scheduler:
                     if victim is r:
                         self._finish(r, "out_of_pages")
                         dropped.append(r)
+                        recount()
                     break
                 self._preempt(victim)
                 preempted.append(victim)
-                free = list(self.cache.num_free_pages())
-                for s in segments:  # pages already promised to this step's segments
-                    for g, x in enumerate(self._needed(s.request, s.count)):
-                        free[g] -= x
+                recount()
                 if victim is r:
                     break
             if id(r) in planned:

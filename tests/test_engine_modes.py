@@ -1,0 +1,104 @@
+"""The engine against the plain implementation, for every way of cutting and batching:
+each request alone and whole; most of it in one step and the last 32 tokens one by one;
+portions of changing size down to two tokens; and mixed, up to four live requests with
+portions of some beside single tokens of others and so few pages that they are used again
+(the pool is poisoned with NaN, so a stale or foreign page shows).
+
+On the CPU the engine runs with the plain PyTorch ops (this checks cache, batch and step
+logic); on the GPU with the HIP kernels, in float32 and bfloat16.  In bfloat16 the plain
+implementation is given the engine's expert choices: a near-tie in the router may fall
+the other way under rounding, which is no fault; that such flips happen only at near-ties
+is checked separately."""
+import pytest
+import torch
+
+import traces
+from jax_llm_examples_amd.engine.replay import make_runner
+from plain_llama4 import PlainModel
+from tiny_configs import TINY
+
+LENGTHS = {"A": [1, 80, 33, 47, 64, 9], "B": [120, 2, 49, 96, 31, 77], "C": [61, 40, 5, 83]}
+MODES = {"whole": traces.whole, "tail": traces.tail, "portions": traces.portions, "mixed": traces.mixed}
+TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}  # of the largest logit of the request
+
+
+def _vocab(name):
+    c = TINY[name]
+    return c.get("text_config", c)["vocab_size"]
+
+
+def _check(name, folder, dtype, device, mode, reference_ops):
+    lengths = LENGTHS[name] + (LENGTHS[name][::-1] + LENGTHS[name] if mode == "mixed" else [])
+    reqs = traces.random_requests(_vocab(name), lengths, seed=5)
+    steps = MODES[mode](reqs)
+    runner = make_runner(folder, dtype, traces.max_live_tokens(steps), device, reference_ops=reference_ops,
+                         poison=True)
+    got, routes = traces.run_trace(runner, steps, record_routing=True)
+    if mode == "mixed":  # so few pages that they were used again
+        assert all(g.pool.handed_out > g.pool.num_pages for g in runner.cache.groups)
+    runner.cache.check()
+    assert runner.cache.num_live() == 0 and all(g.pool.num_held == 0 for g in runner.cache.groups)
+    plain = PlainModel(folder)
+    worst = 0.0
+    for rid, toks in reqs.items():
+        forced = routes.get(rid) if dtype == "bfloat16" else None
+        info = {}
+        ref = plain.logits(toks, forced=forced, info=info)
+        assert got[rid].shape == ref.shape
+        assert torch.isfinite(got[rid]).all(), f"{rid}: non-finite logits (a page that was given back?)"
+        err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
+        bad = (err > TOL[dtype]).nonzero().squeeze(-1).tolist()
+        assert not bad, f"{name} {dtype} {mode} {rid}: first wrong position {bad[0]} of {len(toks)}, error {err[bad[0]]:.3g}"
+        worst = max(worst, float(err.max()))
+        if dtype == "float32" and rid in routes:  # float32: the same experts, always
+            for li, (idx, _) in info.items():
+                assert torch.equal(routes[rid][li].long(), idx), f"{rid} layer {li}: expert choice differs"
+    return worst
+
+
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(TINY))
+def test_cpu_plain_ops_float32(model_dirs, name, mode):
+    _check(name, model_dirs[name], "float32", "cpu", mode, reference_ops=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(TINY))
+def test_gpu_float32(model_dirs, name, mode):
+    _check(name, model_dirs[name], "float32", "cuda:0", mode, reference_ops=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+@pytest.mark.parametrize("name", list(TINY))
+def test_gpu_bfloat16(model_dirs_bf16, name, mode):
+    _check(name, model_dirs_bf16[name], "bfloat16", "cuda:0", mode, reference_ops=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(TINY))
+def test_gpu_bfloat16_expert_choices_differ_only_at_near_ties(model_dirs_bf16, name):
+    folder = model_dirs_bf16[name]
+    reqs = traces.random_requests(_vocab(name), LENGTHS[name], seed=5)
+    steps = traces.portions(reqs)
+    runner = make_runner(folder, "bfloat16", traces.max_live_tokens(steps), "cuda:0")
+    _, routes = traces.run_trace(runner, steps, record_routing=True)
+    plain = PlainModel(folder)
+    total = flips = 0
+    for rid, toks in reqs.items():
+        info = {}
+        plain.logits(toks, forced=routes[rid], info=info)  # same inputs to every router as the engine's run
+        for li, (_, scores) in info.items():
+            k = routes[rid][li].shape[1]
+            top = torch.sort(scores, dim=-1, descending=True)
+            want = top.indices[:, :k]
+            got = routes[rid][li].long()
+            diff = (got != want).any(-1)
+            total += diff.numel()
+            flips += int(diff.sum())
+            if diff.any():
+                # where the choice differs, the scores of the two candidates are close
+                margin = (torch.gather(scores, 1, want) - torch.gather(scores, 1, got)).abs().max(-1).values
+                assert (margin[diff] < 0.05 * scores.std()).all(), f"{rid} layer {li}: a clear choice went wrong"
+    assert flips <= 0.05 * total

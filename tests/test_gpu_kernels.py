@@ -1,0 +1,299 @@
+"""Each HIP kernel alone against its plain PyTorch statement (ops/reference.py), at sizes
+other than the engine tests' models: widths and vocabularies that are no power of two,
+head sizes in steps of 16, odd head counts and groups."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DT = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from jax_llm_examples_amd.engine import get_ops
+    return get_ops(DEV)
+
+
+@pytest.fixture(scope="module")
+def ref():
+    from jax_llm_examples_amd.ops.reference import ReferenceOps
+    return ReferenceOps()
+
+
+def _tol(dt):
+    return dict(rtol=2e-5, atol=2e-6) if dt == torch.float32 else dict(rtol=1.6e-2, atol=1e-3)
+
+
+def _rand(*shape, dt=torch.float32, scale=1.0, seed=None):
+    g = torch.Generator(device="cpu").manual_seed(seed if seed is not None else hash(shape) % 1000)
+    return (torch.randn(*shape, generator=g) * scale).to(dt).to(DEV)
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_embed(ops, ref, dt):
+    table = _rand(311, 80, dt=dt)
+    tok = torch.tensor([0, 310, 5, 5, 17], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.embed(tok, table), ref.embed(tok, table))
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("d", [80, 1000, 5120])
+def test_add_rmsnorm(ops, ref, dt, d):
+    for delta_dt, weighted, want32 in [(None, True, False), (dt, True, True), (torch.float32, False, True)]:
+        x = _rand(7, d, seed=1)
+        delta = None if delta_dt is None else _rand(7, d, dt=delta_dt, seed=2)
+        w = _rand(d, seed=3) if weighted else None
+        x1, x2 = x.clone(), x.clone()
+        h1, h32_1 = ops.add_rmsnorm(x1, delta, w, 1e-3, dt, want32)
+        h2, h32_2 = ref.add_rmsnorm(x2, delta, w, 1e-3, dt, want32)
+        assert torch.allclose(x1, x2, rtol=1e-6, atol=1e-6)  # the residual is updated in place, float32
+        assert torch.allclose(h1.float(), h2.float(), **_tol(dt))
+        if want32:
+            assert torch.allclose(h32_1, h32_2, rtol=2e-5, atol=2e-6)
+            assert h32_1.dtype == torch.float32
+
+
+def test_rmsnorm_eps_is_inside_the_root(ops):
+    x = torch.full((1, 64), 1e-3, device=DEV)
+    h, _ = ops.add_rmsnorm(x, None, None, 1e-2, torch.float32)
+    assert torch.allclose(h, torch.full_like(h, 1e-3 / math.sqrt(1e-6 + 1e-2)), rtol=1e-5)
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_silu_mul_gather_add(ops, ref, dt):
+    gu = _rand(9, 2 * 56, dt=dt, scale=3.0)
+    assert torch.allclose(ops.silu_mul(gu).float(), ref.silu_mul(gu).float(), **_tol(dt))
+    x = _rand(11, 90, dt=dt)
+    idx = torch.tensor([10, 0, 3, 3], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.gather_rows(x, idx), x[idx.long()])
+    r, d = _rand(11, 90, seed=4), _rand(11, 90, dt=dt, seed=5)
+    want = r + d.float()
+    ops.add_residual(r, d)
+    assert torch.allclose(r, want, rtol=1e-6, atol=1e-6)
+
+
+def _prep_case(hq, hk, dh, n, ps, dt, seed=0):
+    qkv = _rand(n, (hq + 2 * hk) * dh, dt=dt, seed=seed)
+    pos = torch.randint(0, 500, (n,), generator=torch.Generator().manual_seed(seed)).to(torch.int32).to(DEV)
+    pages = 2 * n // ps + 3
+    slots = torch.randperm(pages * ps, generator=torch.Generator().manual_seed(seed + 1))[:n].to(torch.int32).to(DEV)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, dh, 2).float() / dh))).to(DEV)
+    return qkv, pos, pages, slots, inv_freq
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("hq,hk,dh", [(4, 2, 16), (5, 1, 48), (40, 8, 128), (3, 3, 256), (6, 2, 80)])
+def test_qk_prepare_kv_write(ops, ref, dt, hq, hk, dh):
+    n, ps = 13, 8
+    qkv, pos, pages, slots, inv_freq = _prep_case(hq, hk, dh, n, ps, dt)
+    for rope, eps, qs in [(True, 1e-5, None), (False, None, (16.0, 0.1)), (True, None, None), (False, None, None),
+                          (True, 1e-3, (4.0, 0.3))]:
+        c1 = torch.zeros(pages, 2, hk, ps, dh, dtype=dt, device=DEV)
+        c2 = c1.clone()
+        q1 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq if rope else None, eps, qs, c1, slots)
+        q2 = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq if rope else None, eps, qs, c2, slots)
+        assert torch.allclose(q1.float(), q2.float(), **_tol(dt))
+        assert torch.allclose(c1.float(), c2.float(), **_tol(dt))
+        assert (c1[:, 1] != 0).any() and torch.equal(c1 == 0, c2 == 0)  # wrote exactly the same places
+    q3 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq, None, None, None, None)  # a run that only reads
+    assert torch.allclose(q3.float(), ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq, None, None, None,
+                                                               None).float(), **_tol(dt))
+
+
+def test_rotation_angles_are_float32_at_large_positions(ops):
+    # the angle must be pos * inv_freq in float32: with a bfloat16 position 257 becomes 256
+    dh = 16
+    qkv = torch.zeros(1, 3 * dh, device=DEV)
+    qkv[0, 0] = 1.0
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, dh, 2).float() / dh))).to(DEV)
+    for p in (257, 4099, 131071):
+        pos = torch.tensor([p], dtype=torch.int32, device=DEV)
+        q = ops.qk_prepare_kv_write(qkv, 1, 1, dh, pos, inv_freq, None, None, None, None)
+        assert abs(float(q[0, 0, 0]) - math.cos(float(torch.tensor(float(p)) * inv_freq[0].cpu()))) < 2e-6
+        assert abs(float(q[0, 0, 1]) - math.sin(float(torch.tensor(float(p)) * inv_freq[0].cpu()))) < 2e-6
+
+
+def _attention_case(hq, hk, dh, ps, dt, seg_specs, seed=0):
+    """seg_specs: (tokens already in the cache, new tokens) per segment; pages are scattered."""
+    g = torch.Generator().manual_seed(seed)
+    total_pages = sum(-(-(a + b) // ps) for a, b in seg_specs) + 5
+    perm = torch.randperm(total_pages, generator=g).tolist()
+    kv = (torch.randn(total_pages, 2, hk, ps, dh, generator=g) * 0.7).to(dt).to(DEV)
+    width = max(-(-(a + b) // ps) for a, b in seg_specs)
+    bt = torch.full((len(seg_specs), width), -1, dtype=torch.int32)
+    pos, seg = [], []
+    for i, (a, b) in enumerate(seg_specs):
+        for j in range(-(-(a + b) // ps)):
+            bt[i, j] = perm.pop()
+        pos += list(range(a, a + b))
+        seg += [i] * b
+    n = len(pos)
+    q = (torch.randn(n, hq, dh, generator=g)).to(dt).to(DEV)
+    return (q, kv, bt.to(DEV), torch.tensor(pos, dtype=torch.int32, device=DEV),
+            torch.tensor(seg, dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("hq,hk,dh,ps", [(4, 2, 16, 16), (5, 1, 48, 16), (6, 3, 32, 8), (8, 8, 64, 16),
+                                         (10, 2, 128, 16), (2, 1, 256, 32), (3, 1, 80, 16)])
+@pytest.mark.parametrize("retention", [("all",), ("chunk", 24), ("window", 37)])
+def test_paged_attention(ops, ref, dt, hq, hk, dh, ps, retention):
+    case = _attention_case(hq, hk, dh, ps, dt, [(0, 70), (130, 1), (45, 9), (63, 2), (200, 1)])
+    q, kv, bt, pos, seg = case
+    got = ops.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
+    want = ref.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
+    tol = dict(rtol=2e-5, atol=2e-6) if dt == torch.float32 else dict(rtol=1.6e-2, atol=4e-3)
+    assert torch.allclose(got.float(), want.float(), **tol)
+
+
+def test_attention_refuses_a_head_size_it_cannot_do(ops):
+    from jax_llm_examples_amd.ops.hip import KernelError
+    q, kv, bt, pos, seg = _attention_case(2, 1, 20, 16, torch.float32, [(0, 4)])
+    with pytest.raises(KernelError, match="refuses"):
+        ops.paged_attention(q, kv, bt, pos, seg, ("all",), 1.0)
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_attention_finds_one_far_key_among_hundreds_and_respects_the_window_edge(ops, dt):
+    """Random weights would hide a key that is skipped: here one key's score stands out, so the
+    output is that key's value, if and only if the rule lets the query see it."""
+    hq, hk, dh, ps = 2, 1, 32, 16
+    T = 700
+    q, kv, bt, pos, seg = _attention_case(hq, hk, dh, ps, dt, [(T - 1, 1)], seed=3)
+    q.zero_()
+    q[0, :, 0] = 8.0
+
+    def run(hot, retention):
+        k = kv.clone()
+        k[:, 0] *= 0.05
+        page, off = int(bt[0, hot // ps]), hot % ps
+        k[page, 0, 0, off, 0] = 8.0  # score 64 * scale, far above the rest
+        k[page, 1, 0, off] = 3.0  # its value
+        return ops.paged_attention(q, k, bt, pos, seg, retention, 1.0).float()
+
+    for hot in (3, 15, 16, 17, 333, T - 2):  # page edges among them
+        assert torch.allclose(run(hot, ("all",)), torch.full((1, hq * dh), 3.0, device=DEV), atol=2e-2)
+    C = 96  # the query at 699 is in the chunk that starts at 672
+    assert torch.allclose(run(672, ("chunk", C)), torch.full((1, hq * dh), 3.0, device=DEV), atol=2e-2)
+    assert run(671, ("chunk", C)).abs().max() < 1.0  # one before the chunk: not seen
+    W = 100  # window: keys 600..699
+    assert torch.allclose(run(600, ("window", W)), torch.full((1, hq * dh), 3.0, device=DEV), atol=2e-2)
+    assert run(599, ("window", W)).abs().max() < 1.0
+
+
+def test_attention_reading_a_page_that_was_given_back_is_not_silent(ops):
+    q, kv, bt, pos, seg = _attention_case(2, 1, 16, 16, torch.float32, [(40, 1)])
+    bt[0, 1] = -1
+    out = ops.paged_attention(q, kv, bt, pos, seg, ("all",), 1.0)
+    assert torch.isnan(out).all()
+
+
+@pytest.mark.parametrize("n,d,e,k", [(50, 5120, 16, 1), (7, 80, 3, 2), (33, 96, 128, 4), (1, 64, 4, 1)])
+def test_moe_route(ops, ref, n, d, e, k):
+    h, w = _rand(n, d, seed=1), _rand(e, d, scale=0.05, seed=2)
+    ids, gates, logits = ops.moe_route(h, w, k, want_logits=True)
+    rid, rg = ref.moe_route(h, w, k)
+    assert torch.allclose(logits, h @ w.t(), rtol=1e-4, atol=1e-5)
+    assert torch.equal(ids, rid) and torch.allclose(gates, rg, rtol=1e-5, atol=1e-6)
+
+
+def test_moe_route_lowest_index_wins_ties(ops):
+    h = _rand(5, 64, seed=1)
+    w = _rand(1, 64, seed=2).expand(6, 64).contiguous()  # every expert the same score
+    ids, gates = ops.moe_route(h, w, 3)
+    assert ids.tolist() == [[0, 1, 2]] * 5
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("n,d,f,e,k", [(50, 96, 40, 16, 1), (9, 80, 56, 3, 2), (130, 64, 24, 5, 1), (1, 64, 32, 4, 1)])
+def test_moe_experts(ops, ref, dt, n, d, f, e, k):
+    h = _rand(n, d, dt=dt, seed=1)
+    wgu, wd = _rand(e, 2 * f, d, dt=dt, scale=0.2, seed=2), _rand(e, d, f, dt=dt, scale=0.2, seed=3)
+    shared = _rand(n, d, dt=dt, seed=4)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(n)]).to(torch.int32).to(DEV)
+    if e > 3:
+        ids[ids == 2] = 0  # an expert nobody chose
+    gates = torch.rand(n, k, generator=g).to(DEV)
+    got = ops.moe_experts(h, ids, gates, wgu, wd, shared)
+    want = ref.moe_experts(h, ids, gates, wgu, wd, shared)
+    assert got.dtype == torch.float32
+    assert torch.allclose(got, want, **_tol(dt))
+    assert torch.allclose(ops.moe_experts(h, ids, gates, wgu, wd, None), ref.moe_experts(h, ids, gates, wgu, wd, None),
+                          **_tol(dt))
+
+
+def test_moe_align_is_a_stable_grouping(ops):
+    g = torch.Generator().manual_seed(0)
+    ids = torch.randint(0, 7, (300, 2), generator=g).to(torch.int32).to(DEV)
+    gates = torch.rand(300, 2, generator=g).to(DEV)
+    off, tok, gate, inv = ops.moe_align(ids, gates, 7)
+    flat = ids.flatten().cpu()
+    off, tok, gate, inv = off.cpu(), tok.cpu(), gate.cpu(), inv.cpu()
+    assert off[0] == 0 and off[-1] == 600
+    for e in range(7):
+        rows = (flat == e).nonzero().squeeze(-1)
+        assert off[e + 1] - off[e] == rows.numel()
+        assert torch.equal(inv[rows], torch.arange(int(off[e]), int(off[e + 1]), dtype=torch.int32))  # in order
+        assert torch.equal(tok[off[e]: off[e + 1]], (rows // 2).to(torch.int32))
+    assert torch.equal(gate[inv.long()], gates.flatten().cpu())
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_product_kernel_and_lm_head(ops, ref, dt):
+    a, b = _rand(33, 52, dt=dt, seed=1), _rand(70, 52, dt=dt, seed=2)
+    assert torch.allclose(ops.gemm(a, b).float(), ref.linear(a, b).float(), **_tol(dt))
+    h, w = _rand(5, 80, dt=dt, seed=3), _rand(311, 80, dt=dt, seed=4)
+    got = ops.lm_head(h, w)
+    assert got.dtype == torch.float32 and got.shape == (5, 311)
+    assert torch.allclose(got, ref.lm_head(h, w), rtol=2e-5, atol=2e-5)  # float32 accumulation and output
+    assert torch.allclose(ops.linear(h, w).float(), ref.linear(h, w).float(), **_tol(dt))
+
+
+def test_float32_products_are_true_float32(ops):
+    # a reduced-precision matrix mode (tf32/xf32: 10 mantissa bits) would lose the small term
+    a = torch.tensor([[1.0, 2.0 ** -14]], device=DEV).repeat(4, 64)  # 128 columns
+    b = torch.ones(8, 128, device=DEV)
+    want = 64 * (1.0 + 2.0 ** -14)
+    for out in (ops.linear(a, b), ops.lm_head(a, b), ops.gemm(a, b)):
+        assert torch.allclose(out, torch.full_like(out, want), rtol=1e-7)
+
+
+def test_sampling(ops, ref):
+    g = torch.Generator().manual_seed(0)
+    V = 1000
+    logits = torch.randn(6, V, generator=g).to(DEV)
+    logits[0, 17] = logits[0, 400] = 9.0  # two equal maxima: the lower id
+    z = torch.zeros(6, dtype=torch.int32, device=DEV)
+    greedy = ops.sample(logits, torch.zeros(6, device=DEV), z, z, z)
+    assert greedy.tolist() == torch.argmax(logits, -1).tolist() and greedy[0] == 17
+    temp = torch.tensor([0.0, 0.7, 1.0, 1.3, 1.0, 1.0], device=DEV)
+    topk = torch.tensor([0, 0, 5, 16, 1, 0], dtype=torch.int32, device=DEV)
+    seeds = torch.tensor([1, 2, 3, 4, 5, 6], dtype=torch.int32, device=DEV)
+    for c in range(4):
+        ctr = torch.full((6,), c, dtype=torch.int32, device=DEV)
+        got = ops.sample(logits, temp, topk, seeds, ctr)
+        want = ref.sample(logits.cpu(), temp.cpu(), topk.cpu(), seeds.cpu(), ctr.cpu())
+        assert got.tolist() == want.tolist()
+        assert got[4] == torch.argmax(logits[4])  # top_k = 1 is greedy
+        assert int(got[2]) in torch.topk(logits[2], 5).indices.tolist()
+    # a request's draw does not depend on what else is in the batch
+    alone = ops.sample(logits[3:4].contiguous(), temp[3:4].contiguous(), topk[3:4].contiguous(),
+                       seeds[3:4].contiguous(), torch.tensor([2], dtype=torch.int32, device=DEV))
+    ctr = torch.full((6,), 2, dtype=torch.int32, device=DEV)
+    assert alone[0] == ops.sample(logits, temp, topk, seeds, ctr)[3]
+
+
+def test_sampling_frequencies_follow_softmax(ops):
+    p = torch.tensor([0.5, 0.25, 0.15, 0.07, 0.03])
+    n = 4000
+    logits = torch.log(p)[None].repeat(n, 1).to(DEV) * 2.0  # temperature 2 undoes the factor
+    out = ops.sample(logits, torch.full((n,), 2.0, device=DEV), torch.zeros(n, dtype=torch.int32, device=DEV),
+                     torch.arange(n, dtype=torch.int32, device=DEV), torch.zeros(n, dtype=torch.int32, device=DEV))
+    freq = torch.bincount(out.cpu().long(), minlength=5).float() / n
+    sigma = torch.sqrt(p * (1 - p) / n)
+    assert ((freq - p).abs() < 4 * sigma).all(), (freq, p)

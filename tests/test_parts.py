@@ -1,0 +1,257 @@
+"""Each part of a layer alone against the plain implementation's function for it, and the
+openness of the design: a toy mixer with state of its own, a toy architecture, a layer
+that runs twice and a layer that reads another layer's cache - all defined here, registered
+and stepped without a change to the framework's files.  Runs with the plain ops on the CPU
+and with the HIP kernels on the GPU."""
+import dataclasses
+import os
+
+import pytest
+import torch
+from safetensors.torch import load_file
+
+import plain_llama4 as P
+import traces
+from jax_llm_examples_amd.cache import CacheManager, CacheView
+from jax_llm_examples_amd.config import ModelPlan, OrderEntry, LayerSpec, part, register_architecture
+from jax_llm_examples_amd.engine import ModelRunner, StepEntry, build_context, get_ops, load_model
+from jax_llm_examples_amd.parts import (CacheNeed, DecoderModel, Mixer, ParamSpec, build_feed_forward, build_mixer,
+                                        build_norm, register_mixer)
+from jax_llm_examples_amd.parts.residual import Residual
+from jax_llm_examples_amd.weights import TensorBinding, init_random_
+from tiny_configs import tiny_config_json
+
+DEVICES = [pytest.param("cpu", id="cpu-plain-ops"), pytest.param("cuda:0", id="gpu-hip", marks=pytest.mark.gpu)]
+
+
+def _ops(device):
+    return get_ops(device, reference_ops=(device == "cpu"))
+
+
+def _ctx_for(ops, device, cache, cuts, vocab=512):
+    """Contexts for one request 'r' fed in the given cuts (list of token lists)."""
+    for toks in cuts:
+        if not cache.has_request("r"):
+            cache.add_request("r")
+        cache.reserve("r", len(toks))
+        yield build_context(ops, torch.float32, device, cache, [StepEntry("r", toks, [])], vocab)
+        cache.commit("r")
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,layer", [("A", 0), ("A", 3), ("B", 1), ("B", 2), ("C", 0), ("C", 1)])
+def test_attention_part_alone(model_dirs, device, name, layer):
+    """Rotary + chunked and NoPE + temperature layers: the mixer over the paged cache, whole and in
+    portions, equals the plain attention block on the whole sequence."""
+    folder = model_dirs[name]
+    cfg = P.read_config(folder)
+    w = P.read_weights(folder)
+    model = load_model(folder, "float32", device)
+    mixer = model.blocks[layer].mixer
+    ops = _ops(device)
+    T = 75
+    x = torch.randn(T, cfg["hidden_size"], generator=torch.Generator().manual_seed(1))
+    want = P.attention_block(x, w, f"model.layers.{layer}.", cfg, layer, torch.arange(T))
+    for sizes in ([T], [30, 2, 17, 1, 1, 24]):
+        cache = CacheManager({0: mixer.cache_need()}, page_size=16, num_pages=8, max_requests=1,
+                             dtype=torch.float32, device=device, poison=True)
+        outs, o = [], 0
+        cuts = [[0] * n for n in sizes]
+        for ctx, n in zip(_ctx_for(ops, device, cache, cuts), sizes):
+            g = ctx.groups[0]
+            view = CacheView(0, True, kv=cache.groups[0].tensors[0], block_table=g.block_table,
+                             slot_mapping=g.slot_mapping, attn_meta=g, group=0)
+            outs.append(mixer.forward(x[o:o + n].to(device), ctx, view).cpu())
+            o += n
+        got = torch.cat(outs)
+        assert torch.allclose(got, want, rtol=1e-4, atol=2e-6), (got - want).abs().max()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name,layer", [("A", 1), ("B", 0), ("B", 3), ("C", 0), ("C", 1)])
+def test_feed_forward_part_alone(model_dirs, device, name, layer):
+    folder = model_dirs[name]
+    cfg = P.read_config(folder)
+    w = P.read_weights(folder)
+    model = load_model(folder, "float32", device)
+    ff = model.blocks[layer].feed_forward
+    ops = _ops(device)
+    x = torch.randn(41, cfg["hidden_size"], generator=torch.Generator().manual_seed(2))
+    p = f"model.layers.{layer}.feed_forward."
+    if layer in cfg["moe_layers"]:
+        want, idx, _ = P.moe_block(x, w, p, cfg)
+    else:
+        want = P.mlp_block(x, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+
+    @dataclasses.dataclass
+    class Ctx:
+        ops: object
+        record_routing: bool = True
+        forced_routing: dict = None
+
+    xd = x.to(device)
+    got = ff.forward(xd, xd if ff.wants_float32_input else None, Ctx(ops)).float().cpu()
+    assert torch.allclose(got, want, rtol=1e-4, atol=2e-6)
+    if layer in cfg["moe_layers"]:
+        assert torch.equal(ff.last_routing[0].cpu().long(), idx)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_norm_part_and_residual(device):
+    ops = _ops(device)
+    norm = build_norm(part("rmsnorm", eps=1e-4, weighted=True, size=80))
+    norm.allocate(torch.float32, torch.device(device))
+    norm.params["weight"].copy_(torch.randn(80, generator=torch.Generator().manual_seed(3)))
+
+    @dataclasses.dataclass
+    class Ctx:
+        ops: object
+        dtype: torch.dtype = torch.float32
+
+    x = torch.randn(6, 80, generator=torch.Generator().manual_seed(4))
+    d = torch.randn(6, 80, generator=torch.Generator().manual_seed(5))
+    res = Residual(x.clone().to(device))
+    res.add(d.to(device))
+    h, h32 = norm.forward(res, Ctx(ops), want32=True)
+    want = P.rms_norm(x + d, norm.params["weight"].cpu(), 1e-4)
+    assert torch.allclose(h.cpu(), want, rtol=1e-5, atol=1e-6) and torch.allclose(h32.cpu(), want, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(res.x.cpu(), x + d) and res.pending is None
+    with pytest.raises(AssertionError):
+        res.add(d.to(device)), res.add(d.to(device))
+
+
+def test_unknown_kinds_are_named():
+    with pytest.raises(KeyError, match="unknown mixer kind 'conv'.*attention"):
+        build_mixer(part("conv"))
+    with pytest.raises(KeyError, match="unknown feed-forward kind"):
+        build_feed_forward(part("glu2"))
+
+
+# ----------------------------------------------------------------------------- a toy mixer with state
+@register_mixer("toy_decayed_sum")
+class ToyDecayedSum(Mixer):
+    """``s_t = decay * s_{t-1} + h_t``; output ``W s_t``.  Its state per request is ``s`` (one vector):
+    no pages at all.  Written with plain PyTorch: it is a toy that lives in this test."""
+
+    def __init__(self, spec):
+        super().__init__()
+        self.hidden, self.decay = int(spec.hidden_size), float(spec.decay)
+
+    def param_specs(self):
+        return {"w": ParamSpec((self.hidden, self.hidden))}
+
+    def cache_need(self):
+        return CacheNeed(kv=None, state_shape=(self.hidden,), state_dtype=torch.float32)
+
+    def forward(self, h, ctx, cache):
+        out = torch.empty_like(h)
+        slots = ctx.state_slots.tolist()
+        o = 0
+        for seg, n in enumerate(ctx.seg_lens):
+            s = cache.state[slots[seg]]
+            for t in range(n):
+                s = self.decay * s + h[o + t].float()
+                out[o + t] = (self.params["w"].float() @ s).to(h.dtype)
+            cache.state[slots[seg]] = s
+            o += n
+        return out
+
+
+class ToyArchitecture:
+    names = ("ToyForCausalLM",)
+
+    def parse_config(self, top):
+        return dict(top)
+
+    def config_to_dict(self, cfg, architecture=None):
+        return dict(cfg)
+
+    def plan(self, cfg):
+        D = cfg["hidden_size"]
+        norm = part("rmsnorm", eps=1e-5, weighted=True, size=D)
+        toy = LayerSpec(mixer=part("toy_decayed_sum", hidden_size=D, decay=cfg["decay"]),
+                        feed_forward=part("dense_swiglu", hidden_size=D, intermediate_size=cfg["intermediate_size"]),
+                        mixer_norm=norm, feed_forward_norm=norm)
+        attn = LayerSpec(mixer=part("attention", hidden_size=D, num_heads=2, num_kv_heads=1, head_dim=16,
+                                    softmax_scale=0.25, position=part("rope_interleaved", theta=100.0, scaling=None),
+                                    qk_norm=None, retention=("window", 11), query_scale=None),
+                         feed_forward=part("moe_sigmoid_shared", hidden_size=D, num_experts=3, top_k=2,
+                                           intermediate_size=24, shared_intermediate_size=0),
+                         mixer_norm=norm, feed_forward_norm=norm)
+        # layer 1 (attention) runs twice, the second time with a cache of its own; then layer 0 again with new
+        # state; the last run reads the keys and values that the first run of layer 1 wrote
+        order = (OrderEntry(0, 0), OrderEntry(1, 1), OrderEntry(1, 2), OrderEntry(0, 3),
+                 OrderEntry(1, 1, writes_cache=False))
+        return ModelPlan(vocab_size=cfg["vocab_size"], hidden_size=D, layers=(toy, attn), order=order,
+                         final_norm=norm)
+
+    def bindings(self, cfg, plan):
+        return []
+
+
+register_architecture(ToyArchitecture())
+
+
+def _toy_model(device):
+    from jax_llm_examples_amd.config import get_architecture
+    arch = get_architecture("ToyForCausalLM")
+    cfg = arch.parse_config({"hidden_size": 48, "intermediate_size": 40, "vocab_size": 97, "decay": 0.8})
+    model = DecoderModel(arch.plan(cfg), torch.float32, device)
+    model.allocate()
+    init_random_(model, seed=4, std=0.2)
+    return model
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_toy_mixer_with_state_runs_and_does_not_depend_on_the_cut(device):
+    model = _toy_model(device)
+    needs = model.cache_needs()
+    assert needs[0].kv is None and needs[0].state_shape == (48,) and needs[1].retention == ("window", 11)
+    reqs = traces.random_requests(97, [50, 23, 41], seed=2)
+    results = {}
+    for mode in ("whole", "portions", "mixed"):
+        steps = getattr(traces, mode)(reqs)
+        cache = CacheManager(needs, page_size=4, num_pages=40, max_requests=3, dtype=torch.float32, device=device,
+                             poison=True)
+        assert set(cache.state) == {0, 3} and cache.state[0].shape == (3, 48)
+        assert [g.cache_ids for g in cache.groups] == [[1, 2]]
+        runner = ModelRunner(model, cache, _ops(device))
+        results[mode] = traces.run_trace(runner, steps)
+        cache.check()
+        assert all(g.pool.num_held == 0 for g in cache.groups)
+    for rid in reqs:
+        assert torch.isfinite(results["whole"][rid]).all()
+        assert torch.allclose(results["portions"][rid], results["whole"][rid], rtol=1e-4, atol=1e-5)
+        assert torch.allclose(results["mixed"][rid], results["whole"][rid], rtol=1e-4, atol=1e-5)
+    # the state does what the mixer says: against a direct evaluation of the first run
+    toks = reqs["r1"]
+    x = model.embed.params["weight"][torch.tensor(toks)].float().cpu()
+    h = P.rms_norm(x, model.blocks[0].mixer_norm.params["weight"].cpu(), 1e-5)
+    s, outs = torch.zeros(48), []
+    for t in range(len(toks)):
+        s = 0.8 * s + h[t]
+        outs.append(model.blocks[0].mixer.params["w"].float().cpu() @ s)
+    direct = torch.stack(outs)
+
+    @dataclasses.dataclass
+    class Ctx:
+        ops: object
+        state_slots: torch.Tensor
+        seg_lens: list
+
+    state = torch.zeros(1, 48, device=device)
+    got = model.blocks[0].mixer.forward(h.to(device), Ctx(_ops(device), torch.tensor([0]), [len(toks)]),
+                                        CacheView(0, True, state=state))
+    assert torch.allclose(got.cpu(), direct, rtol=1e-4, atol=1e-5)
+
+
+def test_order_is_checked():
+    norm = part("rmsnorm", eps=1e-5, weighted=True, size=8)
+    layer = LayerSpec(part("toy_decayed_sum", hidden_size=8, decay=0.5),
+                      part("dense_swiglu", hidden_size=8, intermediate_size=8), norm, norm)
+    with pytest.raises(ValueError, match="both write cache 0"):
+        ModelPlan(10, 8, (layer,), (OrderEntry(0, 0), OrderEntry(0, 0)), norm)
+    with pytest.raises(ValueError, match="reads cache 1 before"):
+        ModelPlan(10, 8, (layer,), (OrderEntry(0, 0), OrderEntry(0, 1, writes_cache=False)), norm)
+    with pytest.raises(ValueError, match="names layer 3"):
+        ModelPlan(10, 8, (layer,), (OrderEntry(3, 0),), norm)

@@ -1,0 +1,334 @@
+"""Pins the plain implementation (tests/plain_llama4.py) by what fixes it beside the
+reference's text: library special cases and invariants, each chosen so that a plausible
+mistake (a wrong sign or pairing, eps outside the root, a norm in the wrong place) fails.
+The reference holds no stored vectors for these formulas (its tests assert nothing
+numeric, ``llama4/tests/test_model.py:129-143``); its kernel self-tests give the semantics
+of a key window ``[start, length)`` (``llama4/llama4_jax/ragged_attention.py:251-286``) and a
+1e-4 relative bound for the grouped product (``decode_ragged_dot.py:338``).
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_llama4 as P
+
+torch.manual_seed(0)
+
+
+# ----------------------------------------------------------------------------- rms norm
+def test_rms_norm_is_the_library_routine():
+    x = torch.randn(5, 24, dtype=torch.float64)
+    g = torch.randn(24, dtype=torch.float64)
+    for eps in (1e-5, 1e-2, 0.5):  # a large eps shows eps outside the root or added to rms
+        assert torch.allclose(P.rms_norm(x, g, eps), F.rms_norm(x, (24,), g, eps), atol=1e-12)
+        assert torch.allclose(P.rms_norm(x, None, eps), F.rms_norm(x, (24,), None, eps), atol=1e-12)
+
+
+def test_rms_norm_unit_rms_and_scale_invariance():
+    x = torch.randn(7, 32, dtype=torch.float64)
+    y = P.rms_norm(x, None, 0.0)
+    assert torch.allclose(y.pow(2).mean(-1), torch.ones(7, dtype=torch.float64))
+    assert torch.allclose(P.rms_norm(3.7 * x, None, 0.0), y)
+    g = torch.full((32,), 2.0, dtype=torch.float64)  # weight used as it is, not 1 + weight
+    assert torch.allclose(P.rms_norm(x, g, 0.0), 2.0 * y)
+
+
+# ----------------------------------------------------------------------------- rotary
+def _rope(x, pos, theta=10000.0, scaling=None):
+    freq = P.rope_frequencies(x.shape[-1], theta, scaling, x.dtype)
+    sin, cos = P.rope_sin_cos(pos, freq)
+    return P.apply_rope(x, sin, cos)
+
+
+def test_rope_is_complex_multiplication_of_adjacent_pairs():
+    T, H, dh = 9, 3, 16
+    x = torch.randn(T, H, dh, dtype=torch.float64)
+    pos = torch.arange(T) * 3 + 1
+    freq = P.rope_frequencies(dh, 10000.0, None, torch.float64)
+    ang = pos.double()[:, None] * freq[None, :]
+    want = torch.view_as_real(torch.view_as_complex(x.reshape(T, H, dh // 2, 2)) *
+                              torch.polar(torch.ones_like(ang), ang)[:, None, :]).reshape(T, H, dh)
+    assert torch.allclose(_rope(x, pos), want, atol=1e-12)
+
+
+def test_rope_frequencies_formula():
+    f = P.rope_frequencies(8, 10000.0, None, torch.float64)
+    want = torch.tensor([10000.0 ** (-2 * j / 8) for j in range(4)], dtype=torch.float64)
+    assert torch.allclose(f, want, rtol=1e-6)
+
+
+def test_rope_identity_at_zero_norm_preserving_and_relative():
+    T, dh = 6, 16
+    q = torch.randn(1, 1, dh, dtype=torch.float64)
+    k = torch.randn(1, 1, dh, dtype=torch.float64)
+    assert torch.allclose(_rope(q, torch.zeros(1, dtype=torch.long)), q)
+    for p in (1, 17, 300):
+        assert torch.allclose(_rope(q, torch.tensor([p])).norm(), q.norm())
+    # <R(p) q, R(p') k> depends on p - p' only: a wrong sign in one of the two lines breaks it
+    def dot(pq, pk):
+        return (_rope(q, torch.tensor([pq])) * _rope(k, torch.tensor([pk]))).sum()
+    assert torch.allclose(dot(5, 2), dot(105, 102), atol=1e-10)
+    assert torch.allclose(dot(40, 47), dot(0, 7), atol=1e-10)
+    assert not torch.allclose(dot(5, 2), dot(5, 3), atol=1e-6)
+
+
+def test_rope_pairs_are_adjacent_not_half_split():
+    dh = 8
+    x = torch.zeros(1, 1, dh, dtype=torch.float64)
+    x[0, 0, 0] = 1.0  # first element of pair 0
+    y = _rope(x, torch.tensor([1]))
+    # rotation by angle 1 * freq[0] = 1 rad mixes elements 0 and 1 (adjacent), not 0 and dh/2
+    assert torch.allclose(y[0, 0, 0], torch.tensor(math.cos(1.0), dtype=torch.float64))
+    assert torch.allclose(y[0, 0, 1], torch.tensor(math.sin(1.0), dtype=torch.float64))
+    assert y[0, 0, dh // 2] == 0
+
+
+def test_llama3_scaling_invariants():
+    dh, theta = 64, 500000.0
+    base = P.rope_frequencies(dh, theta, None, torch.float64)
+    one = dict(factor=1.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64)
+    assert torch.allclose(P.rope_frequencies(dh, theta, one, torch.float64), base)
+    sc = dict(factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64)
+    f = P.rope_frequencies(dh, theta, sc, torch.float64)
+    wavelen = 2 * math.pi / base
+    short, long_ = wavelen < 64 / 4.0, wavelen > 64 / 1.0
+    assert short.any() and long_.any() and (~short & ~long_).any()
+    assert torch.allclose(f[short], base[short])
+    assert torch.allclose(f[long_], base[long_] / 4.0)
+    mid = ~short & ~long_
+    assert ((f[mid] <= base[mid] + 1e-12) & (f[mid] >= base[mid] / 4.0 - 1e-12)).all()
+    assert (f[:-1] >= f[1:]).all()  # still decreasing with j
+    # continuous at both edges: a frequency just inside the band is close to the rule outside it
+    def corr(wl):
+        return float(P.llama3_frequency_correction(torch.tensor([2 * math.pi / wl], dtype=torch.float64),
+                                                   4.0, 1.0, 4.0, 64)[0] * wl / (2 * math.pi))
+    assert abs(corr(16.0001) - 1.0) < 1e-4 and abs(corr(63.9999) - 0.25) < 1e-4
+    eq = dict(factor=16.0, low_freq_factor=1.0, high_freq_factor=1.0, original_max_position_embeddings=8192)
+    g = P.rope_frequencies(128, theta, eq, torch.float64)
+    assert torch.isfinite(g).all()
+    b = P.rope_frequencies(128, theta, None, torch.float64)
+    wl = 2 * math.pi / b
+    assert torch.allclose(g[wl > 8192], b[wl > 8192] / 16.0) and torch.allclose(g[wl <= 8192], b[wl <= 8192])
+
+
+# ----------------------------------------------------------------------------- attention
+def _qkv(T, hq, hk, dh):
+    return (torch.randn(T, hq, dh, dtype=torch.float64), torch.randn(T, hk, dh, dtype=torch.float64),
+            torch.randn(T, hk, dh, dtype=torch.float64))
+
+
+def _sdpa(q, k, v, causal=True):
+    o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                       is_causal=causal, enable_gqa=True)
+    return o[0].transpose(0, 1).reshape(q.shape[0], -1)
+
+
+@pytest.mark.parametrize("hq,hk", [(4, 2), (6, 3), (5, 1), (3, 3)])
+def test_attention_without_chunk_is_the_library_routine(hq, hk):
+    T, dh = 13, 16
+    q, k, v = _qkv(T, hq, hk, dh)
+    pos = torch.arange(T)
+    got = P.attention(q, k, v, P.attention_mask(pos, pos, None), dh ** -0.5)
+    assert torch.allclose(got, _sdpa(q, k, v), atol=1e-10)
+    # a chunk at least as long as the sequence changes nothing
+    got2 = P.attention(q, k, v, P.attention_mask(pos, pos, 64), dh ** -0.5)
+    assert torch.allclose(got2, got)
+
+
+def test_attention_one_head_without_mask_is_softmax_qk_v():
+    T, dh = 7, 8
+    q, k, v = _qkv(T, 1, 1, dh)
+    full = torch.ones(T, T, dtype=torch.bool)
+    got = P.attention(q, k, v, full, dh ** -0.5)
+    want = torch.softmax(q[:, 0] @ k[:, 0].T / math.sqrt(dh), -1) @ v[:, 0]
+    assert torch.allclose(got, want, atol=1e-12)
+
+
+def test_gqa_is_repeating_kv_heads():
+    T, dh = 9, 8
+    q, k, v = _qkv(T, 6, 2, dh)
+    pos = torch.arange(T)
+    m = P.attention_mask(pos, pos, None)
+    a = P.attention(q, k, v, m, 0.3)
+    b = P.attention(q, k.repeat_interleave(3, 1), v.repeat_interleave(3, 1), m, 0.3)
+    assert torch.allclose(a, b, atol=1e-12)  # head h uses kv head h // 3, not h % 2
+
+
+def test_chunked_attention_is_the_library_routine_per_chunk():
+    T, dh, C = 23, 16, 8
+    q, k, v = _qkv(T, 4, 2, dh)
+    pos = torch.arange(T)
+    got = P.attention(q, k, v, P.attention_mask(pos, pos, C), dh ** -0.5)
+    for s in range(0, T, C):
+        e = min(T, s + C)
+        assert torch.allclose(got[s:e], _sdpa(q[s:e], k[s:e], v[s:e]), atol=1e-10)
+
+
+def test_attention_is_causal_and_rows_are_convex_combinations():
+    T, dh = 10, 8
+    q, k, v = _qkv(T, 2, 2, dh)
+    pos = torch.arange(T)
+    m = P.attention_mask(pos, pos, None)
+    a = P.attention(q, k, v, m, 1.0)
+    k2, v2 = k.clone(), v.clone()
+    k2[6:] += 5.0
+    v2[6:] -= 3.0
+    assert torch.allclose(P.attention(q, k2, v2, m, 1.0)[:6], a[:6])
+    ones = torch.ones_like(v)
+    assert torch.allclose(P.attention(q, k, ones, m, 1.0), torch.ones(T, 2 * dh, dtype=torch.float64))
+
+
+def test_key_window_semantics_of_the_reference_decode_kernel():
+    # ragged_attention.py:251-286: a query sees keys in [start, length); here start = chunk start
+    S, dh = 40, 8
+    q = torch.randn(1, 2, dh, dtype=torch.float64)
+    k, v = torch.randn(S, 1, dh, dtype=torch.float64), torch.randn(S, 1, dh, dtype=torch.float64)
+    qpos, C = torch.tensor([S - 1]), 16
+    mask = P.attention_mask(qpos, torch.arange(S), C)
+    start = (S - 1) // C * C
+    assert mask[0].tolist() == [start <= i < S for i in range(S)]
+    got = P.attention(q, k, v, mask, 0.5)
+    full = torch.ones(1, S - start, dtype=torch.bool)
+    assert torch.allclose(got, P.attention(q, k[start:], v[start:], full, 0.5))
+
+
+def test_temperature_scale():
+    pos = torch.arange(100)
+    s = P.temperature_scale(pos, 16.0, 0.1, torch.float64)
+    assert (s[:15] == 1).all() and s[15] > 1  # 1 until pos + 1 reaches floor_scale
+    steps = (s[1:] != s[:-1]).nonzero().squeeze(-1) + 1
+    assert all((int(p) + 1) % 16 == 0 for p in steps)  # it changes only where pos + 1 is a multiple
+    assert torch.allclose(s[47], torch.tensor(1 + 0.1 * math.log(1 + 3), dtype=torch.float64))
+    assert (P.temperature_scale(pos, 8192.0, 0.1) == 1).all()
+    # scaling the query equals scaling that row of scores
+    q, k, v = _qkv(1, 1, 1, 8)
+    k5, v5 = torch.randn(5, 1, 8, dtype=torch.float64), torch.randn(5, 1, 8, dtype=torch.float64)
+    full = torch.ones(1, 5, dtype=torch.bool)
+    assert torch.allclose(P.attention(q * 1.7, k5, v5, full, 0.5), P.attention(q, k5, v5, full, 0.5 * 1.7))
+
+
+# ----------------------------------------------------------------------------- feed-forward
+def test_mlp_block_is_swiglu():
+    x = torch.randn(4, 12, dtype=torch.float64)
+    wg, wu, wd = (torch.randn(20, 12, dtype=torch.float64), torch.randn(20, 12, dtype=torch.float64),
+                  torch.randn(12, 20, dtype=torch.float64))
+    want = F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd)
+    assert torch.allclose(P.mlp_block(x, wg, wu, wd), want, atol=1e-12)
+    assert not torch.allclose(P.mlp_block(x, wu, wg, wd), want, atol=1e-6)  # gate and up are not alike
+
+
+def test_route_is_topk_then_sigmoid():
+    x = torch.randn(11, 16, dtype=torch.float64)
+    w = torch.randn(6, 16, dtype=torch.float64)
+    gates, idx, scores = P.route(x, w, 2)
+    tv, ti = torch.topk(x @ w.T, 2)
+    assert torch.equal(idx, ti) and torch.allclose(gates, torch.sigmoid(tv))
+    assert torch.allclose(gates[:, 0], torch.sigmoid(x @ w.T).max(-1).values)  # no softmax, no renormalising
+    xt = torch.zeros(1, 16, dtype=torch.float64)  # all scores equal: the lowest index wins
+    assert P.route(xt, w, 2)[1].tolist() == [[0, 1]]
+
+
+def _moe_weights(E, D, Fi, dtype=torch.float64, same=False):
+    w = {
+        "router.weight": torch.randn(E, D, dtype=dtype),
+        "experts.gate_up_proj": torch.randn(E, D, 2 * Fi, dtype=dtype) * 0.3,
+        "experts.down_proj": torch.randn(E, Fi, D, dtype=dtype) * 0.3,
+        "shared_expert.gate_proj.weight": torch.randn(Fi, D, dtype=dtype) * 0.3,
+        "shared_expert.up_proj.weight": torch.randn(Fi, D, dtype=dtype) * 0.3,
+        "shared_expert.down_proj.weight": torch.randn(D, Fi, dtype=dtype) * 0.3,
+    }
+    if same:
+        for k in ("experts.gate_up_proj", "experts.down_proj"):
+            w[k] = w[k][:1].expand(E, -1, -1).contiguous()
+    return w
+
+
+def _routed_only(x, w, cfg):
+    out, idx, _ = P.moe_block(x, w, "", cfg)
+    shared = P.mlp_block(x, w["shared_expert.gate_proj.weight"], w["shared_expert.up_proj.weight"],
+                         w["shared_expert.down_proj.weight"])
+    return out - shared, idx
+
+
+def test_moe_with_equal_experts_is_mlp_of_gated_input_plus_shared():
+    E, D, Fi = 4, 12, 10
+    w = _moe_weights(E, D, Fi, same=True)
+    cfg = {"intermediate_size": Fi, "num_experts_per_tok": 1}
+    x = torch.randn(9, D, dtype=torch.float64)
+    routed, idx = _routed_only(x, w, cfg)
+    g = torch.sigmoid((x @ w["router.weight"].T).max(-1).values)[:, None]
+    gu = w["experts.gate_up_proj"][0]
+    # the gate multiplies the expert's input (not its output): SwiGLU is not linear, so this tells them apart
+    want = P.mlp_block(x * g, gu[:, :Fi].T, gu[:, Fi:].T, w["experts.down_proj"][0].T)
+    assert torch.allclose(routed, want, atol=1e-10)
+    wrong = g * P.mlp_block(x, gu[:, :Fi].T, gu[:, Fi:].T, w["experts.down_proj"][0].T)
+    assert not torch.allclose(routed, wrong, atol=1e-6)
+
+
+def test_moe_is_a_loop_over_experts_with_masked_rows_and_permutation_invariant():
+    E, D, Fi = 5, 8, 6
+    w = _moe_weights(E, D, Fi)
+    cfg = {"intermediate_size": Fi, "num_experts_per_tok": 2}
+    x = torch.randn(14, D, dtype=torch.float64)
+    routed, idx = _routed_only(x, w, cfg)
+    gates = torch.sigmoid(torch.gather(x @ w["router.weight"].T, 1, idx))
+    want = torch.zeros_like(x)
+    for e in range(E):  # the grouped product's own oracle (decode_ragged_dot.py:227-236)
+        for j in range(2):
+            rows = idx[:, j] == e
+            xe = x[rows] * gates[rows, j:j + 1]
+            gu = xe @ w["experts.gate_up_proj"][e]
+            want[rows] += (F.silu(gu[:, :Fi]) * gu[:, Fi:]) @ w["experts.down_proj"][e]
+    assert torch.allclose(routed, want, atol=1e-10)
+    perm = torch.randperm(E)
+    w2 = dict(w)
+    for k in ("router.weight", "experts.gate_up_proj", "experts.down_proj"):
+        w2[k] = w[k][perm]
+    assert torch.allclose(P.moe_block(x, w2, "", cfg)[0], P.moe_block(x, w, "", cfg)[0], atol=1e-10)
+    p = torch.randperm(14)  # token-wise
+    assert torch.allclose(P.moe_block(x[p], w, "", cfg)[0], P.moe_block(x, w, "", cfg)[0][p], atol=1e-10)
+
+
+def test_moe_with_one_expert():
+    D, Fi = 8, 6
+    w = _moe_weights(1, D, Fi)
+    cfg = {"intermediate_size": Fi, "num_experts_per_tok": 1}
+    x = torch.randn(5, D, dtype=torch.float64)
+    routed, idx = _routed_only(x, w, cfg)
+    assert (idx == 0).all()
+    g = torch.sigmoid(x @ w["router.weight"].T)
+    gu = w["experts.gate_up_proj"][0]
+    assert torch.allclose(routed, P.mlp_block(x * g, gu[:, :Fi].T, gu[:, Fi:].T, w["experts.down_proj"][0].T),
+                          atol=1e-10)
+
+
+# ----------------------------------------------------------------------------- whole model
+def test_model_is_causal_and_chunk_local(model_dirs):
+    m = P.PlainModel(model_dirs["A"])
+    t = torch.randint(0, 512, (70,)).tolist()
+    a = m.logits(t)
+    t2 = list(t)
+    t2[50] = (t2[50] + 1) % 512
+    b = m.logits(t2)
+    assert torch.equal(a[:50], b[:50]) and not torch.allclose(a[50:], b[50:])
+
+
+def test_positions_shift_only_matters_through_distances_on_rope_layers(model_dirs):
+    # in a model whose layers are all rotary with no chunk boundary crossed, shifting every position
+    # leaves the logits unchanged; here checked at the level of one attention block
+    cfg = P.read_config(model_dirs["A"])
+    w = P.read_weights(model_dirs["A"], torch.float64)
+    x = torch.randn(10, cfg["hidden_size"], dtype=torch.float64)
+    base = P.attention_block(x, w, "model.layers.0.", cfg, 0, torch.arange(10))
+    shifted = P.attention_block(x, w, "model.layers.0.", cfg, 0, torch.arange(10) + 64)  # same chunk phase
+    assert torch.allclose(base, shifted, atol=1e-9)
+    crossing = P.attention_block(x, w, "model.layers.0.", cfg, 0, torch.arange(10) + 27)  # crosses 32
+    assert not torch.allclose(base, crossing, atol=1e-6)
+    # the NoPE layer ignores positions except through the temperature (floor_scale 16)
+    n0 = P.attention_block(x, w, "model.layers.3.", cfg, 3, torch.arange(10))
+    n1 = P.attention_block(x, w, "model.layers.3.", cfg, 3, torch.arange(10) + 3)
+    assert torch.allclose(n0, n1, atol=1e-12)
+    n2 = P.attention_block(x, w, "model.layers.3.", cfg, 3, torch.arange(10) + 16)
+    assert not torch.allclose(n0, n2, atol=1e-6)
