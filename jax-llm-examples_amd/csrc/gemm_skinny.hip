@@ -1,0 +1,172 @@
+// Weight-streaming matrix product for few rows (decode): bfloat16 in, float32 accumulate on MFMA.
+//
+//   Y[t, n] = scale[t] * sum_k X[arow(t), k] * W[g(t)][n, k]          (plain)
+//   Y[t, f] = silu(s * gate) * (s * up),  gate/up = rows f and F + f of W[g(t)]   (SWIGLU, s = scale[t])
+//
+// The cost is reading W once; the rows of X are few (up to 16 * MT per group and block).  The
+// weights are the MFMA's A operand (16 weight rows x 32 k per instruction, each lane reads 16
+// contiguous bytes of a weight row), the activations its B operand (16 tokens), so no data is
+// transposed.  A block is 4 wavefronts that split K between them (k-blocks of 32 interleaved, so
+// together they read 256 contiguous bytes of each weight row) and add their partial sums in
+// shared memory in a fixed order.  Each block owns two 16-row weight tiles (SWIGLU: the gate tile
+// and its up tile, so the activation is formed in the epilogue); grid = (row tiles, token tiles,
+// groups); blocks of groups without rows leave at once.
+#include "common.h"
+
+using namespace jle;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
+  const uint4 v = *reinterpret_cast<const uint4*>(p);
+  return __builtin_bit_cast(bf16x8, v);
+}
+__device__ __forceinline__ bf16x8 zero8() {
+  const uint4 v = {0u, 0u, 0u, 0u};
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+template <typename OutT>
+__device__ __forceinline__ void store_out(OutT* p, float v);
+template <>
+__device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
+template <>
+__device__ __forceinline__ void store_out<bf16_t>(bf16_t* p, float v) { *p = float_to_bf16(v); }
+
+constexpr int kUnroll = 4;
+
+template <int MT, bool SWIGLU, typename OutT>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+                                                          OutT* __restrict__ Y, const int* __restrict__ offsets,
+                                                          const int* __restrict__ a_rows,
+                                                          const float* __restrict__ scale, int M, int Nout, int K) {
+  __shared__ float red[4][2 * MT * 4][64];
+  const int e = blockIdx.z;
+  int row_lo = 0, row_hi = M;
+  if (offsets != nullptr) {
+    row_lo = offsets[e];
+    row_hi = offsets[e + 1];
+  }
+  const int tok0 = row_lo + blockIdx.y * (16 * MT);
+  if (tok0 >= row_hi) return;  // the whole block
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const bf16_t* We = W + (size_t)e * Nout * K;
+  const int half = Nout >> 1;
+  const int base = SWIGLU ? blockIdx.x * 16 : blockIdx.x * 32;  // first output column of the block
+  int ra0, ra1;  // the weight rows this lane reads
+  if (SWIGLU) {
+    ra0 = min(base + r, half - 1);
+    ra1 = half + ra0;
+  } else {
+    ra0 = min(base + r, Nout - 1);
+    ra1 = min(base + 16 + r, Nout - 1);
+  }
+  const bf16_t* a0 = We + (size_t)ra0 * K + g * 8;
+  const bf16_t* a1 = We + (size_t)ra1 * K + g * 8;
+  const bf16_t* xb[MT];
+  bool xv[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int t = tok0 + mt * 16 + r;
+    xv[mt] = t < row_hi;
+    const int src = xv[mt] ? (a_rows != nullptr ? a_rows[t] : t) : 0;
+    xb[mt] = X + (size_t)src * K + g * 8;
+  }
+  f32x4 acc0[MT], acc1[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    acc0[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc1[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int nkb = (K + 31) >> 5;
+  for (int kb0 = wave; kb0 < nkb; kb0 += 4 * kUnroll) {
+    bf16x8 A0[kUnroll], A1[kUnroll], B[kUnroll][MT];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int kb = kb0 + 4 * u;
+      const bool ok = kb < nkb && (kb * 32 + g * 8) < K;  // K is a multiple of 8
+      A0[u] = ok ? load8(a0 + kb * 32) : zero8();
+      A1[u] = ok ? load8(a1 + kb * 32) : zero8();
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) B[u][mt] = (ok && xv[mt]) ? load8(xb[mt] + kb * 32) : zero8();
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        acc0[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A0[u], B[u][mt], acc0[mt], 0, 0, 0);
+        acc1[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[u], B[u][mt], acc1[mt], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      red[wave][(0 * MT + mt) * 4 + i][lane] = acc0[mt][i];
+      red[wave][(1 * MT + mt) * 4 + i][lane] = acc1[mt][i];
+    }
+  }
+  __syncthreads();
+  // wavefront w finishes element i = w of every tile: D[row 4 * g + i of the tile][token r]
+  const int i = wave;
+  const int m = g * 4 + i;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      v0 += red[w][(0 * MT + mt) * 4 + i][lane];
+      v1 += red[w][(1 * MT + mt) * 4 + i][lane];
+    }
+    const int t = tok0 + mt * 16 + r;
+    if (t >= row_hi) continue;
+    const float sc = scale != nullptr ? scale[t] : 1.f;
+    if (SWIGLU) {
+      const int f = base + m;
+      if (f < half) {
+        const float gate = v0 * sc, up = v1 * sc;
+        store_out<OutT>(Y + (size_t)t * half + f, gate / (1.0f + expf(-gate)) * up);
+      }
+    } else {
+      const int c0 = base + m, c1 = base + 16 + m;
+      if (c0 < Nout) store_out<OutT>(Y + (size_t)t * Nout + c0, v0 * sc);
+      if (c1 < Nout) store_out<OutT>(Y + (size_t)t * Nout + c1, v1 * sc);
+    }
+  }
+}
+
+// X [*, K] bf16, W [G, Nout, K] bf16, Y [M, Nout] (or [M, Nout / 2] with swiglu) bf16 or float32.
+// max_rows: the most rows any group can have (M if unknown).
+JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* offsets, const int* a_rows,
+                            const float* scale, int swiglu, int out_f32, int M, int Nout, int K, int G, int max_rows,
+                            hipStream_t s) {
+  if (M <= 0 || Nout <= 0) return 0;
+  if (K <= 0 || K % 8 || G < 1 || G > 65535 || (swiglu && Nout % 2)) return JLE_BAD_ARG;
+  if (max_rows <= 0 || max_rows > M) max_rows = M;
+  const int mt = (offsets == nullptr && max_rows > 32) ? 4 : (offsets == nullptr && max_rows > 16) ? 2 : 1;
+  const int ytiles = (max_rows + 16 * mt - 1) / (16 * mt);
+  if (ytiles > 65535) return JLE_BAD_ARG;
+  const int xtiles = swiglu ? (Nout / 2 + 15) / 16 : (Nout + 31) / 32;
+  dim3 g(xtiles, ytiles, G), b(256);
+#define LAUNCH(MT, SW, OT)                                                                                     \
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, SW, OT>), g, b, 0, s, (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, \
+                     offsets, a_rows, scale, M, Nout, K)
+#define PICK(SW, OT)              \
+  do {                            \
+    if (mt == 1) LAUNCH(1, SW, OT); \
+    else if (mt == 2) LAUNCH(2, SW, OT); \
+    else LAUNCH(4, SW, OT);       \
+  } while (0)
+  if (swiglu) {
+    if (out_f32) PICK(true, float); else PICK(true, bf16_t);
+  } else {
+    if (out_f32) PICK(false, float); else PICK(false, bf16_t);
+  }
+#undef PICK
+#undef LAUNCH
+  JLE_LAUNCH_CHECK();
+  return 0;
+}

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
 
@@ -162,9 +163,32 @@ class HipOps:
                    1 if (out_f32 or a.dtype == torch.float32) else 0, m, nout, k, g)
         return out
 
+    SKINNY_MAX_ROWS = 64  # up to here a product is a stream of the weights: the MFMA weight-streaming kernel
+
+    def gemm_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None):
+        """bfloat16 weight-streaming product on MFMA for few rows (see ``gemm_skinny.hip``); with ``swiglu`` the
+        result is ``silu(gate) * up`` of the two halves of ``b``'s rows."""
+        if b.dim() == 2:
+            b = b.unsqueeze(0)
+        g, nout, k = b.shape
+        m = rows if rows is not None else (a_rows.numel() if a_rows is not None else a.shape[0])
+        self._chk(a, torch.bfloat16, None, "A")
+        self._chk(b, torch.bfloat16, None, "B")
+        if a.shape[1] != k:
+            raise KernelError(f"inner sizes differ: A {tuple(a.shape)}, B {tuple(b.shape)}")
+        if k % 8:
+            raise KernelError(f"the MFMA product needs an inner size that is a multiple of 8, got {k}")
+        out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
+                          device=a.device)
+        self._call("jle_gemm_skinny", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
+                   int(out_f32), m, nout, k, g, m)
+        return out
+
     def lm_head(self, h, w):
         if h.dtype == torch.float32:
             return torch.matmul(h, w.t())
+        if h.shape[0] <= self.SKINNY_MAX_ROWS and h.shape[1] % 8 == 0:
+            return self.gemm_skinny(h, w, out_f32=True)
         return self.gemm(h, w, out_f32=True)
 
     def silu_mul(self, gate_up):
@@ -243,9 +267,13 @@ class HipOps:
         e, f2, _ = w_gate_up.shape
         k = expert_ids.shape[1]
         offsets, sorted_token, sorted_gate, inv = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e)
-        gu = self.gemm(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate)
-        act = self.silu_mul(gu)
-        routed = self.gemm(act, w_down, offsets=offsets)
+        if h.dtype == torch.bfloat16 and n * k <= 2 * self.SKINNY_MAX_ROWS and d % 8 == 0 and (f2 // 2) % 8 == 0:
+            act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True)
+            routed = self.gemm_skinny(act, w_down, offsets=offsets)
+        else:
+            gu = self.gemm(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate)
+            act = self.silu_mul(gu)
+            routed = self.gemm(act, w_down, offsets=offsets)
         out = torch.empty(n, d, dtype=torch.float32, device=h.device)
         if shared is not None:
             self._chk(shared, h.dtype, (n, d), "shared expert output")

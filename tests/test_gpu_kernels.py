@@ -303,3 +303,35 @@ def test_sampling_frequencies_follow_softmax(ops):
     freq = torch.bincount(out.cpu().long(), minlength=5).float() / n
     sigma = torch.sqrt(p * (1 - p) / n)
     assert ((freq - p).abs() < 4 * sigma).all(), (freq, p)
+
+
+@pytest.mark.parametrize("m,nout,k", [(1, 64, 64), (8, 70, 104), (16, 33, 32), (17, 96, 40), (40, 500, 264),
+                                       (64, 130, 5120)])
+@pytest.mark.parametrize("out_f32", [False, True])
+def test_weight_streaming_product(ops, ref, m, nout, k, out_f32):
+    a, b = _rand(m, k, dt=torch.bfloat16, seed=1), _rand(nout, k, dt=torch.bfloat16, scale=0.1, seed=2)
+    got = ops.gemm_skinny(a, b, out_f32=out_f32)
+    want = a.float() @ b.float().t()
+    assert got.dtype == (torch.float32 if out_f32 else torch.bfloat16)
+    err = float((got.float() - want).abs().max() / want.abs().max())
+    assert err <= (2e-5 if out_f32 else 5e-3), err  # float32 out: only the order of the sum differs
+
+
+@pytest.mark.parametrize("n,d,f,e,k", [(8, 128, 48, 16, 1), (64, 5120, 64, 16, 1), (20, 264, 40, 3, 2), (3, 64, 24, 128, 1)])
+def test_weight_streaming_product_grouped_with_swiglu(ops, ref, n, d, f, e, k):
+    dt = torch.bfloat16
+    h = _rand(n, d, dt=dt, seed=1)
+    wgu = _rand(e, 2 * f, d, dt=dt, scale=0.1, seed=2)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(n)]).to(torch.int32).to(DEV)
+    if n == 64:
+        ids[:40] = 3  # one expert with more rows than one tile of 16
+    gates = torch.rand(n, k, generator=g).to(DEV)
+    off, tok, gate, inv = ops.moe_align(ids, gates, e)
+    act = ops.gemm_skinny(h, wgu, offsets=off, a_rows=tok, scale=gate, swiglu=True)
+    gu = ops.gemm(h, wgu, offsets=off, a_rows=tok, scale=gate, out_f32=True)  # the general kernel, float32 result
+    want = torch.nn.functional.silu(gu[:, :f]) * gu[:, f:]
+    assert act.shape == (n * k, f)
+    assert float((act.float() - want).abs().max() / want.abs().max()) <= 5e-3
+    plain = ops.gemm_skinny(h, wgu, offsets=off, a_rows=tok, scale=gate, out_f32=True)
+    assert float((plain - gu).abs().max() / gu.abs().max()) <= 2e-5
