@@ -7,6 +7,7 @@
 //   scores: one key per lane (the lane reads its key's row; q is read at a wave-uniform address)
 //   softmax: running maximum and sum across tiles, float32
 //   values: one head element per lane (+64, +128, +192), probabilities broadcast by shuffle
+// Page layout per kv head: keys [page_size][head_dim], values [head_dim][page_size].
 #include "common.h"
 
 using namespace jle;
@@ -64,12 +65,14 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     const bool valid = key >= first && key <= pos;
     float s = -INFINITY;
     const T* krow = nullptr;
+    int voff = 0;
     if (valid) {
       const int page = table[key / ps];
       if (page < 0) {
         bad = true;
       } else {
         krow = kv + (size_t)page * page_stride + head_off + (size_t)(key % ps) * dh;
+        voff = key % ps;
         float dot = 0.f;
         for (int c = 0; c < dh; c += Vec16<T>::kN) {
           Vec16<T> qv, kvv;
@@ -95,11 +98,13 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
       const unsigned long long kaddr = (unsigned long long)krow;
       const unsigned long long kb = __shfl((unsigned long long)kaddr, kk, 64);
       if (kb == 0ull) continue;  // a page that is not there: flagged below
-      const T* vrow = reinterpret_cast<const T*>(kb) + v_off;
+      const int vo = __shfl(voff, kk, 64);
+      // the key's row starts at plane + vo * dh; its value column at plane + v_off + vo
+      const T* vcol = reinterpret_cast<const T*>(kb) - (size_t)vo * dh + v_off + vo;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int d = lane + 64 * i;
-        if (d < dh) acc[i] += pk * Num<T>::load(vrow + d);
+        if (d < dh) acc[i] += pk * Num<T>::load(vcol + (size_t)d * ps);
       }
     }
   }

@@ -1,0 +1,398 @@
+// Paged attention on MFMA (bfloat16 pages, float32 softmax and accumulation), for prefill
+// portions and for decode, head sizes that are multiples of 32 up to 256.
+//
+// One wavefront works on up to 16 * CT *columns* against a range of keys.  A column is a
+// (token, query head) pair: for a prefill tile the columns are consecutive tokens of one segment
+// and one head; for decode they are the query heads that share one kv head, of one token.
+// Everything is kept transposed, so that no operand ever has to be shuffled between lanes:
+//
+//   S^T[key, col] = K[key, :] . Q[col, :]        A = keys (16 rows of the page, as stored),
+//                                                 B = queries (as stored)
+//   softmax over keys: a column lives in the lanes with the same (lane % 16); running max / sum
+//   O^T[d, col]  += V^T[d, key] . P^T[key, col]   A = values, stored transposed in the page
+//                                                 ([head_dim][page_size]); B = the probabilities,
+//                                                 which are already in the lanes that need them
+//
+// The accumulator of 16x16x32 holds, in lane (c = lane % 16, g = lane / 16), rows 4g..4g+3 of
+// column c; the B operand wants 8 k-values for column c in that same lane.  Taking the 32 keys of
+// one step as two tiles of 16 and assigning k-slot (g, j) to key 4g + j of the first tile (j < 4)
+// or of the second (j >= 4) makes the accumulators of S^T the B operand of the second product
+// as they are.  The A operand of that product then reads, for element d, keys 4g..4g+3 of each
+// tile: 8 contiguous bytes of the transposed value page.
+//
+// Decode splits a token's keys into ranges of kSplit absolute positions; each range is one
+// work item and leaves (max, sum, unnormalised O); a second kernel merges them in order.  Which
+// ranges and tiles a query visits depends only on its position and the retention rule.
+#include "common.h"
+
+using namespace jle;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kSplit = 256;  // keys per decode work item
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ int first_key(int mode, int param, int pos) {
+  if (mode == 1) return (pos / param) * param;
+  if (mode == 2) return pos - param + 1 > 0 ? pos - param + 1 : 0;
+  return 0;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+}
+
+struct Columns {  // per lane, for each of its column tiles
+  int token;      // row of q / out
+  int head;       // query head
+  int lo, hi;     // keys this column may read within the wave's range (inclusive); lo > hi: none
+};
+
+// The shared core.  DH: head size; CT: column tiles.  Returns through m, l, acc (O^T, unnormalised).
+template <int DH, int CT>
+__device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv,
+                                       const int* __restrict__ table, const Columns (&col)[CT], int k_lo, int k_hi,
+                                       int hk, int Hq, int Hkv, int ps, float scale_log2, float (&m)[CT],
+                                       float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad) {
+  const int lane = threadIdx.x & 63;
+  const int c16 = lane & 15, g = lane >> 4;
+  constexpr int KC = DH / 32;  // k-steps of the first product
+  constexpr int DT = DH / 16;  // row tiles of O^T
+  const size_t plane = (size_t)ps * DH;
+  const size_t page_stride = 2 * (size_t)Hkv * plane;
+
+  bf16x8 qb[CT][KC];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const bf16_t* qrow = q + ((size_t)col[ct].token * Hq + col[ct].head) * DH + g * 8;
+    const bool ok = col[ct].lo <= col[ct].hi;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      uint4 v = {0u, 0u, 0u, 0u};
+      if (ok) v = *reinterpret_cast<const uint4*>(qrow + c * 32);
+      qb[ct][c] = __builtin_bit_cast(bf16x8, v);
+    }
+    m[ct] = -INFINITY;
+    l[ct] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int kb = (k_lo / 32) * 32; kb <= k_hi; kb += 32) {
+    f32x4 st[CT][2];
+    const bf16_t* vbase[2];
+    bool active[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const int key0 = kb + 16 * tt;
+      active[tt] = key0 <= k_hi && key0 + 15 >= k_lo;
+      int page = -1;
+      if (active[tt]) {
+        page = table[key0 / ps];
+        if (page < 0) {
+          bad = true;
+          active[tt] = false;
+        }
+      }
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      vbase[tt] = nullptr;
+      if (active[tt]) {
+        const bf16_t* kbase = kv + (size_t)page * page_stride + (size_t)hk * plane;
+        const int off = key0 % ps;
+        const bf16_t* krow = kbase + (size_t)(off + c16) * DH + g * 8;
+        vbase[tt] = kbase + (size_t)Hkv * plane + off + 4 * g;  // + d * ps
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+          const uint4 kvv = *reinterpret_cast<const uint4*>(krow + c * 32);
+          const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+            st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
+        }
+      }
+    }
+    // mask, running max and sum per column
+    bf16x8 pb[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      float s[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + 16 * tt + 4 * g + i;
+          const bool ok = active[tt] && key >= col[ct].lo && key <= col[ct].hi;
+          const float v = ok ? st[ct][tt][i] * scale_log2 : -INFINITY;
+          s[tt * 4 + i] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[ct], mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float corr = exp2f(m[ct] - m_use);  // m = -inf: 0 (nothing accumulated yet)
+      float sum = 0.f;
+      float p[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        p[j] = exp2f(s[j] - m_use);  // masked: exp2(-inf) = 0
+        sum += p[j];
+      }
+      sum += __shfl_xor(sum, 16, 64);
+      sum += __shfl_xor(sum, 32, 64);
+      l[ct] = l[ct] * corr + sum;
+      m[ct] = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        acc[ct][dt][0] *= corr;
+        acc[ct][dt][1] *= corr;
+        acc[ct][dt][2] *= corr;
+        acc[ct][dt][3] *= corr;
+      }
+      const uint4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+      pb[ct] = __builtin_bit_cast(bf16x8, pk);
+    }
+    // values: keys outside [k_lo, k_hi] may never have been written: they are read as zero
+    uint32_t keep[2][2];  // per tile, per pair of keys: which halves to keep
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const int key = kb + 16 * tt + 4 * g + 2 * h2;
+        const uint32_t lo_ok = (key >= k_lo && key <= k_hi) ? 0x0000ffffu : 0u;
+        const uint32_t hi_ok = (key + 1 >= k_lo && key + 1 <= k_hi) ? 0xffff0000u : 0u;
+        keep[tt][h2] = lo_ok | hi_ok;
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint4 vv = {0u, 0u, 0u, 0u};
+      const size_t drow = (size_t)(dt * 16 + c16) * ps;
+      if (active[0]) {
+        const uint2 t0 = *reinterpret_cast<const uint2*>(vbase[0] + drow);
+        vv.x = t0.x & keep[0][0];
+        vv.y = t0.y & keep[0][1];
+      }
+      if (active[1]) {
+        const uint2 t1 = *reinterpret_cast<const uint2*>(vbase[1] + drow);
+        vv.z = t1.x & keep[1][0];
+        vv.w = t1.y & keep[1][1];
+      }
+      const bf16x8 a = __builtin_bit_cast(bf16x8, vv);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct], acc[ct][dt], 0, 0, 0);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ prefill portions
+// tiles: [num_tiles][2] = (first token, number of tokens <= 16 * CT), all of one segment.
+// One wavefront per (tile, query head); the heads of one kv head are neighbours.
+template <int DH, int CT>
+__global__ __launch_bounds__(256) void attention_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
+    const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
+    int table_width, const int* __restrict__ tiles, int num_tiles, int ret_mode, int ret_param, float scale_log2,
+    int Hq, int Hkv, int ps) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= num_tiles * Hq) return;
+  const int tile = item / Hq, h = item - tile * Hq;
+  const int n0 = tiles[2 * tile], nt = tiles[2 * tile + 1];
+  const int hk = h / (Hq / Hkv);
+  const int c16 = lane & 15, g = lane >> 4;
+  const int p_first = positions[n0], p_last = p_first + nt - 1;  // consecutive positions of one segment
+  const int k_lo = first_key(ret_mode, ret_param, p_first);  // the rule's start never decreases with the position
+  const int k_hi = p_last;
+  Columns col[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = ct * 16 + c16;
+    const bool ok = c < nt;
+    const int pos = p_first + c;
+    col[ct].token = ok ? n0 + c : n0;
+    col[ct].head = h;
+    col[ct].lo = ok ? first_key(ret_mode, ret_param, pos) : 1;
+    col[ct].hi = ok ? pos : 0;
+  }
+  float m[CT], l[CT];
+  f32x4 acc[CT][DH / 16];
+  bool bad = false;
+  attend<DH, CT>(q, kv, block_table + (size_t)token_segment[n0] * table_width, col, k_lo, k_hi, hk, Hq, Hkv, ps,
+                 scale_log2, m, l, acc, bad);
+  bad = __any(bad);
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    if (ct * 16 + c16 >= nt) continue;
+    const float inv = bad ? __builtin_nanf("") : (l[ct] > 0.f ? 1.0f / l[ct] : 0.f);
+    bf16_t* o = out + ((size_t)col[ct].token * Hq + h) * DH + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt) {
+      const uint2 v = {pack_bf16(acc[ct][dt][0] * inv, acc[ct][dt][1] * inv),
+                       pack_bf16(acc[ct][dt][2] * inv, acc[ct][dt][3] * inv)};
+      *reinterpret_cast<uint2*>(o + dt * 16) = v;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ decode
+// dec_tokens: [num_dec] rows of q that are single decode tokens.  One wavefront per
+// (decode token, kv head, key range); ws_ml: [item][16 * CT][2], ws_o: [item][16 * CT][DH],
+// item = (d * Hkv + hk) * max_splits + split.
+template <int DH, int CT>
+__global__ __launch_bounds__(256) void attention_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, float* __restrict__ ws_ml, float* __restrict__ ws_o,
+    const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
+    int table_width, const int* __restrict__ dec_tokens, int num_dec, int max_splits, int ret_mode, int ret_param,
+    float scale_log2, int Hq, int Hkv, int ps) {
+  const int lane = threadIdx.x & 63;
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= num_dec * Hkv * max_splits) return;
+  const int split = item % max_splits;
+  const int hk = (item / max_splits) % Hkv;
+  const int d = item / (max_splits * Hkv);
+  const int n = dec_tokens[d];
+  const int pos = positions[n];
+  const int first = first_key(ret_mode, ret_param, pos);
+  const int s_abs = first / kSplit + split;
+  if (s_abs > pos / kSplit) return;  // this token has fewer ranges
+  const int k_lo = max(first, s_abs * kSplit), k_hi = min(pos, s_abs * kSplit + kSplit - 1);
+  const int G = Hq / Hkv;
+  const int c16 = lane & 15, g = lane >> 4;
+  Columns col[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = ct * 16 + c16;
+    const bool ok = c < G;
+    col[ct].token = n;
+    col[ct].head = ok ? hk * G + c : hk * G;
+    col[ct].lo = ok ? k_lo : 1;
+    col[ct].hi = ok ? k_hi : 0;
+  }
+  float m[CT], l[CT];
+  f32x4 acc[CT][DH / 16];
+  bool bad = false;
+  attend<DH, CT>(q, kv, block_table + (size_t)token_segment[n] * table_width, col, k_lo, k_hi, hk, Hq, Hkv, ps,
+                 scale_log2, m, l, acc, bad);
+  bad = __any(bad);
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = ct * 16 + c16;
+    if (c >= G) continue;
+    const size_t slot = (size_t)item * (16 * CT) + c;
+    if (g == 0) {
+      ws_ml[slot * 2] = bad ? __builtin_nanf("") : m[ct];
+      ws_ml[slot * 2 + 1] = l[ct];
+    }
+    float* o = ws_o + slot * DH + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DH / 16; ++dt) *reinterpret_cast<f32x4*>(o + dt * 16) = acc[ct][dt];
+  }
+}
+
+// Merges a decode token's key ranges, in order.  One block of DH threads per (decode token, head).
+__global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
+                                              bf16_t* __restrict__ out, const int* __restrict__ positions,
+                                              const int* __restrict__ dec_tokens, int max_splits, int ret_mode,
+                                              int ret_param, int Hq, int Hkv, int DH, int cols) {
+  const int d = blockIdx.x / Hq, h = blockIdx.x % Hq;
+  const int n = dec_tokens[d];
+  const int pos = positions[n];
+  const int first = first_key(ret_mode, ret_param, pos);
+  const int ns = pos / kSplit - first / kSplit + 1;
+  const int G = Hq / Hkv, hk = h / G, c = h - hk * G;
+  const size_t item0 = ((size_t)d * Hkv + hk) * max_splits;
+  float mx = -INFINITY;
+  for (int s = 0; s < ns; ++s) mx = fmaxf(mx, ws_ml[((item0 + s) * cols + c) * 2]);  // NaN (a missing page) stays
+  bool nan = false;
+  float l = 0.f;
+  for (int s = 0; s < ns; ++s) {
+    const float ms = ws_ml[((item0 + s) * cols + c) * 2];
+    nan = nan || ms != ms;
+    if (ms != -INFINITY && ms == ms) l += ws_ml[((item0 + s) * cols + c) * 2 + 1] * exp2f(ms - mx);
+  }
+  for (int e = threadIdx.x; e < DH; e += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < ns; ++s) {
+      const float ms = ws_ml[((item0 + s) * cols + c) * 2];
+      if (ms != -INFINITY && ms == ms) o += ws_o[((item0 + s) * cols + c) * DH + e] * exp2f(ms - mx);
+    }
+    const float r = nan ? __builtin_nanf("") : (l > 0.f ? o / l : 0.f);
+    out[((size_t)n * Hq + h) * DH + e] = float_to_bf16(r);
+  }
+}
+
+static bool head_dim_ok(int dh) { return dh == 32 || dh == 64 || dh == 96 || dh == 128 || dh == 256; }
+
+JLE_API int jle_attention_mfma_supported(int dh, int Hq, int Hkv, int ps) {
+  return head_dim_ok(dh) && Hkv > 0 && Hq % Hkv == 0 && ps >= 16 && ps % 16 == 0;
+}
+
+JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, const int* positions,
+                                  const int* token_segment, const int* block_table, int table_width, const int* tiles,
+                                  int num_tiles, int ret_mode, int ret_param, float scale, int Hq, int Hkv, int dh,
+                                  int ps, hipStream_t s) {
+  if (num_tiles <= 0) return 0;
+  if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps)) return JLE_BAD_ARG;
+  if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
+  const long long items = (long long)num_tiles * Hq;
+  dim3 g((unsigned)((items + 3) / 4)), b(256);
+  const float sl = scale * kLog2e;
+#define LAUNCH(DH)                                                                                                 \
+  hipLaunchKernelGGL((attention_prefill_kernel<DH, 2>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,           \
+                     (bf16_t*)out, positions, token_segment, block_table, table_width, tiles, num_tiles, ret_mode, \
+                     ret_param, sl, Hq, Hkv, ps)
+  switch (dh) {
+    case 32: LAUNCH(32); break;
+    case 64: LAUNCH(64); break;
+    case 96: LAUNCH(96); break;
+    case 128: LAUNCH(128); break;
+    case 256: LAUNCH(256); break;
+  }
+#undef LAUNCH
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
+// ws_ml needs num_dec * Hkv * max_splits * cols * 2 floats, ws_o that many * dh / 2, cols = 16 or 32.
+JLE_API int jle_attention_decode(const void* q, const void* kv, void* out, float* ws_ml, float* ws_o,
+                                 const int* positions, const int* token_segment, const int* block_table,
+                                 int table_width, const int* dec_tokens, int num_dec, int max_splits, int ret_mode,
+                                 int ret_param, float scale, int Hq, int Hkv, int dh, int ps, hipStream_t s) {
+  if (num_dec <= 0) return 0;
+  if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps) || max_splits < 1) return JLE_BAD_ARG;
+  if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
+  const int G = Hq / Hkv;
+  if (G > 32) return JLE_BAD_ARG;
+  const int ct = G > 16 ? 2 : 1;
+  const long long items = (long long)num_dec * Hkv * max_splits;
+  dim3 g((unsigned)((items + 3) / 4)), b(256);
+  const float sl = scale * kLog2e;
+#define LAUNCH(DH, CT)                                                                                              \
+  hipLaunchKernelGGL((attention_decode_kernel<DH, CT>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv, ws_ml,     \
+                     ws_o, positions, token_segment, block_table, table_width, dec_tokens, num_dec, max_splits,     \
+                     ret_mode, ret_param, sl, Hq, Hkv, ps)
+#define PICK(DH)          \
+  do {                    \
+    if (ct == 1) LAUNCH(DH, 1); \
+    else LAUNCH(DH, 2);   \
+  } while (0)
+  switch (dh) {
+    case 32: PICK(32); break;
+    case 64: PICK(64); break;
+    case 96: PICK(96); break;
+    case 128: PICK(128); break;
+    case 256: PICK(256); break;
+  }
+#undef PICK
+#undef LAUNCH
+  JLE_LAUNCH_CHECK();
+  hipLaunchKernelGGL(attention_decode_merge_kernel, dim3(num_dec * Hq), dim3(dh <= 64 ? 64 : 128), 0, s, ws_ml, ws_o,
+                     (bf16_t*)out, positions, dec_tokens, max_splits, ret_mode, ret_param, Hq, Hkv, dh, 16 * ct);
+  JLE_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,6 +1,10 @@
 // After the fused q|k|v projection: rotary embedding over adjacent pairs, weightless
 // L2 (rms) norm of q and k, position-dependent query scale, and the write of k and v
 // into their page.  One wavefront per (token, head); everything in float32.
+//
+// Page layout, per page and kv head: keys [page_size][head_dim] (a key's elements contiguous),
+// values [head_dim][page_size] (one element of all the page's tokens contiguous), so that both
+// are read in the order the attention kernels' matrix instructions take them.
 #include "common.h"
 
 using namespace jle;
@@ -50,20 +54,27 @@ __global__ void qk_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
     mul *= 1.0f + attn_scale * log1pf(floorf(((float)pos + 1.0f) / floor_scale));
   }
   T* dst;
+  size_t stride = 1;  // between consecutive elements of the head
   if (is_q) {
     dst = q_out + ((size_t)n * Hq + h) * dh;
   } else {
     const int slot = slot_mapping[n];
     const int page = slot / page_size, off = slot - page * page_size;
     const int hk = is_v ? h - Hq - Hkv : h - Hq;
-    dst = kv_cache + ((((size_t)page * 2 + (is_v ? 1 : 0)) * Hkv + hk) * page_size + off) * dh;
+    T* plane = kv_cache + (((size_t)page * 2 + (is_v ? 1 : 0)) * Hkv + hk) * page_size * dh;
+    if (is_v) {
+      dst = plane + off;
+      stride = page_size;
+    } else {
+      dst = plane + (size_t)off * dh;
+    }
   }
 #pragma unroll
   for (int i = 0; i < kMaxPairsPerLane; ++i) {
     const int j = lane + 64 * i;
     if (j < half) {
-      Num<T>::store(dst + 2 * j, a[i] * mul);
-      Num<T>::store(dst + 2 * j + 1, b[i] * mul);
+      Num<T>::store(dst + (size_t)(2 * j) * stride, a[i] * mul);
+      Num<T>::store(dst + (size_t)(2 * j + 1) * stride, b[i] * mul);
     }
   }
 }

@@ -29,6 +29,8 @@ class GroupContext:
     slot_mapping: torch.Tensor  # int32 [N]
     width: int
     retention: tuple
+    seg_lens: list = dataclasses.field(default_factory=list)  # host copies, for kernel work lists
+    seg_starts: list = dataclasses.field(default_factory=list)
     meta: dict = dataclasses.field(default_factory=dict)  # kernel launch plans, filled lazily
 
 
@@ -124,7 +126,8 @@ def build_context(ops, dtype, device, cache, entries: Sequence[StepEntry], vocab
     for gi, g in enumerate(cache.groups):
         bt = views[7 + 2 * gi].view(R, group_shapes[gi])
         sm = views[8 + 2 * gi]
-        groups.append(GroupContext(block_table=bt, slot_mapping=sm, width=group_shapes[gi], retention=g.retention))
+        groups.append(GroupContext(block_table=bt, slot_mapping=sm, width=group_shapes[gi], retention=g.retention,
+                                   seg_lens=seg_lens, seg_starts=seg_starts))
     return StepContext(
         ops=ops, dtype=dtype, device=torch.device(device), num_tokens=N, num_segments=R,
         token_ids=token_ids, positions=positions, token_segment=token_segment, cu_seqlens=cu_seqlens,

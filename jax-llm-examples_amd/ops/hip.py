@@ -30,6 +30,9 @@ _SIGNATURES = {
     "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    "jle_attention_mfma_supported": [_i, _i, _i, _i],
+    "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
+    "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
     "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -54,6 +57,7 @@ def load_library():
             fn = getattr(lib, name)
             fn.argtypes = args
             fn.restype = ctypes.c_int
+        lib.jle_attention_mfma_supported.argtypes = [_i, _i, _i, _i]  # a query, not a launch: no stream
         lib._jle_path = path
         _LIB = lib
     return _LIB
@@ -220,6 +224,29 @@ class HipOps:
                    n, hq, hk, dh, max(ps, 1), 0 if kv_cache is None else 1)
         return q
 
+    DECODE_SPLIT = 256  # keys per decode work item (kSplit in attention_mfma.hip)
+    PREFILL_TILE = 32  # tokens per prefill work item
+
+    def attention_plan(self, seg_lens, seg_starts, retention, device):
+        """Work lists of the MFMA attention kernels for one step and one retention rule: the rows that are
+        single decode tokens, and tiles of up to 32 consecutive tokens of longer segments."""
+        from ..parts.base import first_needed_position
+
+        dec, tiles, max_splits = [], [], 1
+        o = 0
+        for n, start in zip(seg_lens, seg_starts):
+            if n == 1:
+                dec.append(o)
+                first = first_needed_position(retention, start)
+                max_splits = max(max_splits, start // self.DECODE_SPLIT - first // self.DECODE_SPLIT + 1)
+            else:
+                for t in range(0, n, self.PREFILL_TILE):
+                    tiles += [o + t, min(self.PREFILL_TILE, n - t)]
+            o += n
+        flat = torch.tensor(dec + tiles, dtype=torch.int32).to(device) if dec or tiles else None
+        return {"num_dec": len(dec), "num_tiles": len(tiles) // 2, "max_splits": max_splits,
+                "dec": flat[: len(dec)] if dec else None, "tiles": flat[len(dec):] if tiles else None}
+
     def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
         n, hq, dh = q.shape
         hk, ps = kv_cache.shape[2], kv_cache.shape[3]
@@ -231,6 +258,37 @@ class HipOps:
         mode = _RET_MODES[retention[0]]
         param = int(retention[1]) if len(retention) > 1 else 0
         out = torch.empty(n, hq * dh, dtype=q.dtype, device=q.device)
+        if (q.dtype == torch.bfloat16 and hq // hk <= 32
+                and self.lib.jle_attention_mfma_supported(dh, hq, hk, ps)):
+            plan = meta.meta.get("attn_plan") if meta is not None else None
+            if plan is None:
+                if meta is not None:
+                    seg_lens, seg_starts = meta.seg_lens, meta.seg_starts
+                else:  # a direct call (tests): recover the segments from the device arrays
+                    seg = token_segment.cpu().tolist()
+                    pos = positions.cpu().tolist()
+                    seg_lens, seg_starts = [], []
+                    for i, sgm in enumerate(seg):
+                        if i == 0 or sgm != seg[i - 1]:
+                            seg_lens.append(0)
+                            seg_starts.append(pos[i])
+                        seg_lens[-1] += 1
+                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device)
+                if meta is not None:
+                    meta.meta["attn_plan"] = plan
+            if plan["num_tiles"]:
+                self._call("jle_attention_prefill", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
+                           _p(block_table), block_table.shape[1], _p(plan["tiles"]), plan["num_tiles"], mode, param,
+                           float(scale), hq, hk, dh, ps)
+            if plan["num_dec"]:
+                cols = 16 if hq // hk <= 16 else 32
+                items = plan["num_dec"] * hk * plan["max_splits"]
+                ws_ml = torch.empty(items * cols * 2, dtype=torch.float32, device=q.device)
+                ws_o = torch.empty(items * cols * dh, dtype=torch.float32, device=q.device)
+                self._call("jle_attention_decode", _p(q), _p(kv_cache), _p(out), _p(ws_ml), _p(ws_o), _p(positions),
+                           _p(token_segment), _p(block_table), block_table.shape[1], _p(plan["dec"]), plan["num_dec"],
+                           plan["max_splits"], mode, param, float(scale), hq, hk, dh, ps)
+            return out
         self._call("jle_paged_attention_generic", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
                    _p(block_table), block_table.shape[1], mode, param, float(scale), self._is_bf16(q), n, hq, hk, dh,
                    ps)

@@ -29,6 +29,12 @@ def retention_start(retention: tuple, pos: torch.Tensor) -> torch.Tensor:
     raise ValueError(f"unknown retention rule {retention!r}")
 
 
+def values_t(kv_cache: torch.Tensor) -> torch.Tensor:
+    """The value planes of the pages as ``[pages, kv_heads, head_dim, page_size]`` (how they lie in memory)."""
+    p, _, hk, ps, dh = kv_cache.shape
+    return kv_cache[:, 1].view(p, hk, dh, ps)  # a view: writes through it land in the cache
+
+
 class ReferenceOps:
     name = "reference"
 
@@ -83,9 +89,10 @@ class ReferenceOps:
         (angle ``pos * inv_freq[j]`` in float32), L2-normalises q and k over the
         head (no weight) if ``qk_norm_eps`` is given, multiplies q by
         ``1 + attn_scale * ln(1 + floor((pos + 1) / floor_scale))`` if
-        ``query_scale = (floor_scale, attn_scale)``, and writes k and v into
-        ``kv_cache[page, 0 | 1, head, offset]`` at ``slot = page * page_size + offset``.
-        Returns q ``[N, num_heads, head_dim]``."""
+        ``query_scale = (floor_scale, attn_scale)``, and writes k and v into their page at
+        ``slot = page * page_size + offset``.  ``kv_cache`` is ``[pages, 2, kv_heads, page_size *
+        head_dim]`` in memory: plane 0 holds keys as ``[page_size, head_dim]``, plane 1 holds values
+        transposed, ``[head_dim, page_size]``.  Returns q ``[N, num_heads, head_dim]``."""
         n = qkv.shape[0]
         dt = qkv.dtype
         hq, hk, dh = num_heads, num_kv_heads, head_dim
@@ -114,7 +121,7 @@ class ReferenceOps:
             page = (slot_mapping // ps).long()
             off = (slot_mapping % ps).long()
             kv_cache[page, 0, :, off] = k.to(kv_cache.dtype)
-            kv_cache[page, 1, :, off] = v.to(kv_cache.dtype)
+            values_t(kv_cache)[page, :, :, off] = v.to(kv_cache.dtype)
         return q.to(dt)
 
     def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
@@ -134,7 +141,7 @@ class ReferenceOps:
                 raise RuntimeError(f"token {i} at position {p} reads a page that was given back")
             off = (kpos % ps).long()
             k = kv_cache[pages, 0, :, off].float()  # [T, hk, dh]
-            v = kv_cache[pages, 1, :, off].float()
+            v = values_t(kv_cache)[pages, :, :, off].float()
             qi = q[i].float().reshape(hk, g, dh)
             sc = torch.einsum("hgd,thd->hgt", qi, k) * scale
             pr = torch.softmax(sc, dim=-1)

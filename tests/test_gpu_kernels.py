@@ -146,10 +146,11 @@ def _attention_case(hq, hk, dh, ps, dt, seg_specs, seed=0):
 
 @pytest.mark.parametrize("dt", DT)
 @pytest.mark.parametrize("hq,hk,dh,ps", [(4, 2, 16, 16), (5, 1, 48, 16), (6, 3, 32, 8), (8, 8, 64, 16),
-                                         (10, 2, 128, 16), (2, 1, 256, 32), (3, 1, 80, 16)])
+                                         (10, 2, 128, 16), (2, 1, 256, 32), (3, 1, 80, 16), (6, 3, 32, 16),
+                                         (40, 8, 128, 16), (20, 1, 96, 48), (4, 4, 256, 16), (5, 5, 64, 64)])
 @pytest.mark.parametrize("retention", [("all",), ("chunk", 24), ("window", 37)])
 def test_paged_attention(ops, ref, dt, hq, hk, dh, ps, retention):
-    case = _attention_case(hq, hk, dh, ps, dt, [(0, 70), (130, 1), (45, 9), (63, 2), (200, 1)])
+    case = _attention_case(hq, hk, dh, ps, dt, [(0, 70), (130, 1), (45, 9), (63, 2), (200, 1), (600, 1), (255, 3)])
     q, kv, bt, pos, seg = case
     got = ops.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
     want = ref.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
@@ -178,7 +179,7 @@ def test_attention_finds_one_far_key_among_hundreds_and_respects_the_window_edge
         k[:, 0] *= 0.05
         page, off = int(bt[0, hot // ps]), hot % ps
         k[page, 0, 0, off, 0] = 8.0  # score 64 * scale, far above the rest
-        k[page, 1, 0, off] = 3.0  # its value
+        k[page, 1, 0].view(dh, ps)[:, off] = 3.0  # its value (values lie transposed in the page)
         return ops.paged_attention(q, k, bt, pos, seg, retention, 1.0).float()
 
     for hot in (3, 15, 16, 17, 333, T - 2):  # page edges among them
