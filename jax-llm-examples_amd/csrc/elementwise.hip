@@ -24,17 +24,81 @@ JLE_API int jle_embed(const int* tok, const void* table, int is_bf16, float* out
 
 // ------------------------------------------------------------------ add + rmsnorm
 // x (float32, the residual) += delta; out = x * rsqrt(mean(x^2) + eps) * weight.
-// One block per row; the sum of squares is formed in a fixed order.
-template <typename DT, typename OT>
-__global__ void add_rmsnorm_kernel(float* __restrict__ x, const DT* __restrict__ delta, const float* __restrict__ w,
-                                   float eps, OT* __restrict__ out, float* __restrict__ out32, int D) {
-  __shared__ float red[4];
-  const size_t base = (size_t)blockIdx.x * D;
+// delta is either a plain tensor or the sum of a token's expert outputs and the shared expert's:
+//   delta[n] = sum_j routed[inv[n * k + j]] + shared[n]
+// One block per row.  Rows up to 8192 wide stay in registers (THREADS * EPT elements); wider rows
+// are read twice.  The sum of squares is formed in a fixed order that depends on the width only.
+template <typename DT>
+struct Delta {
+  const DT* plain;    // [N, D] or null
+  const DT* routed;   // [M, D] or null
+  const int* inv;     // [N * k]
+  const DT* shared;   // [N, D] or null
+  int k;
+  __device__ __forceinline__ bool any() const { return plain != nullptr || routed != nullptr; }
+  __device__ __forceinline__ float at(size_t n, int d, int D) const {
+    float v = 0.f;
+    if (plain != nullptr) v = Num<DT>::load(plain + n * D + d);
+    if (routed != nullptr) {
+      for (int j = 0; j < k; ++j) v += Num<DT>::load(routed + (size_t)inv[n * k + j] * D + d);
+      if (shared != nullptr) v += Num<DT>::load(shared + n * D + d);
+    }
+    return v;
+  }
+};
+
+template <typename DT, typename OT, int THREADS, int EPT>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_reg_kernel(float* __restrict__ x, Delta<DT> delta,
+                                                                  const float* __restrict__ w, float eps,
+                                                                  OT* __restrict__ out, float* __restrict__ out32,
+                                                                  int D) {
+  __shared__ float red[THREADS / 64];
+  const size_t n = blockIdx.x;
+  const size_t base = n * D;
+  float v[EPT];
   float ss = 0.f;
+  const bool add = delta.any();
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) {
+    const int d = threadIdx.x + THREADS * i;
+    v[i] = 0.f;
+    if (d < D) {
+      v[i] = x[base + d];
+      if (add) {
+        v[i] += delta.at(n, d, D);
+        x[base + d] = v[i];
+      }
+      ss += v[i] * v[i];
+    }
+  }
+  const float tot = block_sum<THREADS>(ss, red);
+  const float inv = 1.0f / sqrtf(tot / (float)D + eps);
+#pragma unroll
+  for (int i = 0; i < EPT; ++i) {
+    const int d = threadIdx.x + THREADS * i;
+    if (d < D) {
+      float h = v[i] * inv;
+      if (w != nullptr) h *= w[d];
+      if (out != nullptr) Num<OT>::store(out + base + d, h);
+      if (out32 != nullptr) out32[base + d] = h;
+    }
+  }
+}
+
+template <typename DT, typename OT>
+__global__ __launch_bounds__(256) void add_rmsnorm_wide_kernel(float* __restrict__ x, Delta<DT> delta,
+                                                               const float* __restrict__ w, float eps,
+                                                               OT* __restrict__ out, float* __restrict__ out32,
+                                                               int D) {
+  __shared__ float red[4];
+  const size_t n = blockIdx.x;
+  const size_t base = n * D;
+  float ss = 0.f;
+  const bool add = delta.any();
   for (int d = threadIdx.x; d < D; d += 256) {
     float v = x[base + d];
-    if (delta != nullptr) {
-      v += Num<DT>::load(delta + base + d);
+    if (add) {
+      v += delta.at(n, d, D);
       x[base + d] = v;
     }
     ss += v * v;
@@ -49,18 +113,37 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const DT* __restrict__
   }
 }
 
-JLE_API int jle_add_rmsnorm(float* x, const void* delta, int delta_is_bf16, const float* w, float eps, void* out,
+template <typename DT, typename OT>
+static void launch_add_rmsnorm(float* x, Delta<DT> delta, const float* w, float eps, void* out, float* out32, int N,
+                               int D, hipStream_t s) {
+  dim3 g(N);
+  if (D <= 1024)
+    hipLaunchKernelGGL((add_rmsnorm_reg_kernel<DT, OT, 256, 4>), g, dim3(256), 0, s, x, delta, w, eps, (OT*)out, out32,
+                       D);
+  else if (D <= 8192)
+    hipLaunchKernelGGL((add_rmsnorm_reg_kernel<DT, OT, 1024, 8>), g, dim3(1024), 0, s, x, delta, w, eps, (OT*)out,
+                       out32, D);
+  else
+    hipLaunchKernelGGL((add_rmsnorm_wide_kernel<DT, OT>), g, dim3(256), 0, s, x, delta, w, eps, (OT*)out, out32, D);
+}
+
+// delta_kind: 0 none, 1 plain (delta), 2 expert sum (routed, inv, k, shared)
+JLE_API int jle_add_rmsnorm(float* x, int delta_kind, const void* delta, const void* routed, const int* inv, int k,
+                            const void* shared, int delta_is_bf16, const float* w, float eps, void* out,
                             int out_is_bf16, float* out32, int N, int D, hipStream_t s) {
   if (N <= 0) return 0;
-  dim3 g(N), b(256);
-#define LAUNCH(DT, OT) \
-  hipLaunchKernelGGL((add_rmsnorm_kernel<DT, OT>), g, b, 0, s, x, (const DT*)delta, w, eps, (OT*)out, out32, D)
+#define GO(DT, OT)                                                                              \
+  do {                                                                                          \
+    Delta<DT> dl = {delta_kind == 1 ? (const DT*)delta : nullptr,                               \
+                    delta_kind == 2 ? (const DT*)routed : nullptr, inv, (const DT*)shared, k}; \
+    launch_add_rmsnorm<DT, OT>(x, dl, w, eps, out, out32, N, D, s);                             \
+  } while (0)
   if (delta_is_bf16) {
-    if (out_is_bf16) LAUNCH(bf16_t, bf16_t); else LAUNCH(bf16_t, float);
+    if (out_is_bf16) GO(bf16_t, bf16_t); else GO(bf16_t, float);
   } else {
-    if (out_is_bf16) LAUNCH(float, bf16_t); else LAUNCH(float, float);
+    if (out_is_bf16) GO(float, bf16_t); else GO(float, float);
   }
-#undef LAUNCH
+#undef GO
   JLE_LAUNCH_CHECK();
   return 0;
 }

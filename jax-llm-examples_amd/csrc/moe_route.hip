@@ -6,111 +6,108 @@ using namespace jle;
 
 constexpr int kMaxTopK = 8;
 
-// TPB tokens per block of 256 threads.  logits[e] = sum_d h[d] * W[e][d]: thread t adds the terms
-// d = t, t + 256, ... for 16 experts at a time, then the block adds the threads' sums in a fixed
-// order.  Thread 0 keeps the k best in a sorted list.
-constexpr int kRouteChunk = 16;
-
-template <int TPB>
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ h, const float* __restrict__ w,
-                                                        int* __restrict__ ids, float* __restrict__ gates,
-                                                        float* __restrict__ logits_out, int N, int D, int E, int k) {
-  extern __shared__ float sm[];  // logits [TPB][E], then partial sums [4][TPB][16]
-  float* logits = sm;
-  float* part = sm + TPB * E;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// Router logits: logits[n, e] = sum_d h[n, d] * W[e, d], float32.  One wavefront per expert and
+// TPB tokens; a lane adds the terms of its float4 chunks (chunk = lane, lane + 64, ...) in
+// order, then the lanes' sums are added by a butterfly: the order is the same for any TPB.
+template <int TPB, bool VEC>
+__global__ __launch_bounds__(256) void moe_logits_kernel(const float* __restrict__ h, const float* __restrict__ w,
+                                                         float* __restrict__ logits, int N, int D, int E) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.y * 4 + (threadIdx.x >> 6);
   const int n0 = blockIdx.x * TPB;
-  for (int e0 = 0; e0 < E; e0 += kRouteChunk) {
-    const int ne = E - e0 < kRouteChunk ? E - e0 : kRouteChunk;
-    float acc[TPB][kRouteChunk];
+  if (e >= E) return;
+  const float* we = w + (size_t)e * D;
+  float acc[TPB];
 #pragma unroll
-    for (int t = 0; t < TPB; ++t)
+  for (int t = 0; t < TPB; ++t) acc[t] = 0.f;
+  if (VEC) {  // D is a multiple of 4: rows are 16-byte aligned
+    const int D4 = D >> 2;
+#pragma unroll 4
+    for (int c = lane; c < D4; c += 64) {
+      const float4 wv = *reinterpret_cast<const float4*>(we + 4 * c);
 #pragma unroll
-      for (int j = 0; j < kRouteChunk; ++j) acc[t][j] = 0.f;
-    for (int d = threadIdx.x; d < D; d += 256) {
-      float xv[TPB];
-#pragma unroll
-      for (int t = 0; t < TPB; ++t) xv[t] = (n0 + t < N) ? h[(size_t)(n0 + t) * D + d] : 0.f;
-#pragma unroll
-      for (int j = 0; j < kRouteChunk; ++j) {
-        if (j < ne) {
-          const float wv = w[(size_t)(e0 + j) * D + d];
-#pragma unroll
-          for (int t = 0; t < TPB; ++t) acc[t][j] += xv[t] * wv;
+      for (int t = 0; t < TPB; ++t) {
+        if (n0 + t < N) {
+          const float4 xv = *reinterpret_cast<const float4*>(h + (size_t)(n0 + t) * D + 4 * c);
+          acc[t] += xv.x * wv.x;
+          acc[t] += xv.y * wv.y;
+          acc[t] += xv.z * wv.z;
+          acc[t] += xv.w * wv.w;
         }
       }
     }
+  } else {
+    for (int d = lane; d < D; d += 64) {
+      const float wv = we[d];
 #pragma unroll
-    for (int t = 0; t < TPB; ++t)
-#pragma unroll
-      for (int j = 0; j < kRouteChunk; ++j) {
-        const float v = wave_sum(acc[t][j]);
-        if (lane == 0) part[(wave * TPB + t) * kRouteChunk + j] = v;
-      }
-    __syncthreads();
-    if (threadIdx.x < TPB * kRouteChunk) {
-      const int t = threadIdx.x / kRouteChunk, j = threadIdx.x % kRouteChunk;
-      if (j < ne) {
-        float v = 0.f;
-#pragma unroll
-        for (int wv = 0; wv < 4; ++wv) v += part[(wv * TPB + t) * kRouteChunk + j];
-        logits[t * E + e0 + j] = v;
-      }
+      for (int t = 0; t < TPB; ++t)
+        if (n0 + t < N) acc[t] += h[(size_t)(n0 + t) * D + d] * wv;
     }
-    __syncthreads();
   }
-  if (threadIdx.x < TPB && n0 + threadIdx.x < N) {
-    const int t = threadIdx.x;
-    const size_t n = n0 + t;
-    float best_v[kMaxTopK];
-    int best_i[kMaxTopK];
+#pragma unroll
+  for (int t = 0; t < TPB; ++t) {
+    const float v = wave_sum(acc[t]);
+    if (lane == 0 && n0 + t < N) logits[(size_t)(n0 + t) * E + e] = v;
+  }
+}
+
+// The k largest logits of each token (lowest index first among equals) and their sigmoids.
+__global__ void moe_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids, float* __restrict__ gates,
+                                int N, int E, int k) {
+  const size_t n = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= (size_t)N) return;
+  float best_v[kMaxTopK];
+  int best_i[kMaxTopK];
+#pragma unroll
+  for (int j = 0; j < kMaxTopK; ++j) {
+    best_v[j] = -INFINITY;
+    best_i[j] = -1;
+  }
+  for (int e = 0; e < E; ++e) {
+    float v = logits[n * E + e];
+    // insert into the sorted list; strict '>' keeps the lower index ahead among equals,
+    // and everything behind the insertion point moves down by one
+    int ci = e;
+    bool carrying = false;
 #pragma unroll
     for (int j = 0; j < kMaxTopK; ++j) {
-      best_v[j] = -INFINITY;
-      best_i[j] = -1;
-    }
-    for (int e = 0; e < E; ++e) {
-      float v = logits[t * E + e];
-      if (logits_out != nullptr) logits_out[n * E + e] = v;
-      // insert into the sorted list; strict '>' keeps the lower index ahead among equals,
-      // and everything behind the insertion point moves down by one
-      int ci = e;
-      bool carrying = false;
-#pragma unroll
-      for (int j = 0; j < kMaxTopK; ++j) {
-        if (j < k && (carrying || v > best_v[j] || best_i[j] < 0)) {
-          const float tv = best_v[j];
-          const int ti = best_i[j];
-          best_v[j] = v;
-          best_i[j] = ci;
-          v = tv;
-          ci = ti;
-          carrying = true;
-        }
+      if (j < k && (carrying || v > best_v[j] || best_i[j] < 0)) {
+        const float tv = best_v[j];
+        const int ti = best_i[j];
+        best_v[j] = v;
+        best_i[j] = ci;
+        v = tv;
+        ci = ti;
+        carrying = true;
       }
     }
+  }
 #pragma unroll
-    for (int j = 0; j < kMaxTopK; ++j) {
-      if (j < k) {
-        ids[n * k + j] = best_i[j];
-        gates[n * k + j] = 1.0f / (1.0f + expf(-best_v[j]));
-      }
+  for (int j = 0; j < kMaxTopK; ++j) {
+    if (j < k) {
+      ids[n * k + j] = best_i[j];
+      gates[n * k + j] = 1.0f / (1.0f + expf(-best_v[j]));
     }
   }
 }
 
-JLE_API int jle_moe_route(const float* h, const float* w, int* ids, float* gates, float* logits_out, int N, int D,
-                          int E, int k, hipStream_t s) {
+// logits: [N, E] float32 workspace (also the caller's copy of the router logits)
+JLE_API int jle_moe_route(const float* h, const float* w, int* ids, float* gates, float* logits, int N, int D, int E,
+                          int k, hipStream_t s) {
   if (N <= 0) return 0;
-  if (k < 1 || k > kMaxTopK || k > E || E > 4096) return JLE_BAD_ARG;
-  if (N >= 256) {
-    const size_t smem = (4 * E + 4 * 4 * kRouteChunk) * sizeof(float);
-    hipLaunchKernelGGL(moe_route_kernel<4>, dim3((N + 3) / 4), dim3(256), smem, s, h, w, ids, gates, logits_out, N, D,
-                       E, k);
+  if (k < 1 || k > kMaxTopK || k > E || E > 4096 || logits == nullptr) return JLE_BAD_ARG;
+  const bool vec = D % 4 == 0 && (((uintptr_t)h | (uintptr_t)w) & 15) == 0;
+  const bool many = N >= 64;
+  dim3 g(many ? (N + 7) / 8 : N, (E + 3) / 4), b(256);
+  if (many) {
+    if (vec) hipLaunchKernelGGL((moe_logits_kernel<8, true>), g, b, 0, s, h, w, logits, N, D, E);
+    else hipLaunchKernelGGL((moe_logits_kernel<8, false>), g, b, 0, s, h, w, logits, N, D, E);
   } else {
-    const size_t smem = (E + 4 * kRouteChunk) * sizeof(float);
-    hipLaunchKernelGGL(moe_route_kernel<1>, dim3(N), dim3(256), smem, s, h, w, ids, gates, logits_out, N, D, E, k);
+    if (vec) hipLaunchKernelGGL((moe_logits_kernel<1, true>), g, b, 0, s, h, w, logits, N, D, E);
+    else hipLaunchKernelGGL((moe_logits_kernel<1, false>), g, b, 0, s, h, w, logits, N, D, E);
   }
+  JLE_LAUNCH_CHECK();
+  hipLaunchKernelGGL(moe_topk_kernel, dim3((N + 127) / 128), dim3(128), 0, s, logits, ids, gates, N, E, k);
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -19,7 +19,7 @@ _vp, _i, _f, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_longl
 
 _SIGNATURES = {
     "jle_embed": [_vp, _vp, _i, _vp, _i, _i, _vp],
-    "jle_add_rmsnorm": [_vp, _vp, _i, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
+    "jle_add_rmsnorm": [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
     "jle_add_residual": [_vp, _vp, _i, _ll, _vp],
     "jle_gather_rows": [_vp, _vp, _vp, _i, _i, _vp],
     "jle_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
@@ -39,6 +39,16 @@ _SIGNATURES = {
 
 class KernelError(RuntimeError):
     pass
+
+
+class ExpertSum:
+    """A feed-forward output that is not formed yet: ``sum_j routed[inv[n * k + j]] + shared[n]``.  The kernel
+    that adds it to the residual and norms the result reads the pieces directly."""
+
+    def __init__(self, routed, inv, k: int, shared, n: int, d: int) -> None:
+        self.routed, self.inv, self.k, self.shared = routed, inv, k, shared
+        self.shape = torch.Size((n, d))
+        self.dtype = routed.dtype
 
 
 _LIB = None
@@ -123,22 +133,39 @@ class HipOps:
     def add_rmsnorm(self, x, delta, weight, eps: float, out_dtype, want32: bool = False):
         n, d = x.shape
         self._chk(x, torch.float32, (n, d), "residual")
-        if delta is not None:
+        kind, plain, routed, inv, k, shared, is_bf16 = 0, None, None, None, 0, None, 0
+        if isinstance(delta, ExpertSum):
+            kind, routed, inv, k, shared = 2, delta.routed, delta.inv, delta.k, delta.shared
+            is_bf16 = self._is_bf16(routed)
+        elif delta is not None:
             self._chk(delta, None, (n, d), "branch output")
+            kind, plain, is_bf16 = 1, delta, self._is_bf16(delta)
         if weight is not None:
             self._chk(weight, torch.float32, (d,), "norm weight")
         out = torch.empty(n, d, dtype=out_dtype, device=x.device)
         out32 = torch.empty(n, d, dtype=torch.float32, device=x.device) if want32 else None
-        self._call("jle_add_rmsnorm", _p(x), _p(delta), 0 if delta is None else self._is_bf16(delta), _p(weight),
+        self._call("jle_add_rmsnorm", _p(x), kind, _p(plain), _p(routed), _p(inv), k, _p(shared), is_bf16, _p(weight),
                    float(eps), _p(out), self._is_bf16(out), _p(out32), n, d)
         return out, out32
 
+    def materialize(self, delta):
+        """The tensor an :class:`ExpertSum` stands for (float32)."""
+        if not isinstance(delta, ExpertSum):
+            return delta
+        n, d = delta.shape
+        out = torch.empty(n, d, dtype=torch.float32, device=delta.routed.device)
+        self._call("jle_moe_combine", _p(delta.routed), _p(delta.inv), _p(delta.shared), _p(out),
+                   self._is_bf16(delta.routed), n, delta.k, d)
+        return out
+
     def add_residual(self, x, delta) -> None:
+        delta = self.materialize(delta)
         self._chk(x, torch.float32, None, "residual")
         self._chk(delta, None, x.shape, "branch output")
         self._call("jle_add_residual", _p(x), _p(delta), self._is_bf16(delta), x.numel())
 
     def gather_rows(self, x, idx):
+        x = self.materialize(x)
         m = idx.numel()
         self._chk(x, None, None, "rows")
         self._chk(idx, torch.int32, (m,), "row indices")
@@ -148,9 +175,19 @@ class HipOps:
 
     # ------------------------------------------------------------------ matrix products
     def linear(self, h, w, out_dtype=None):
-        """``h @ w.T`` through the BLAS library (float32: true float32)."""
+        """``h @ w.T``.  Few bfloat16 rows: the weight-streaming MFMA kernel; otherwise the BLAS library
+        (float32: true float32)."""
+        if (h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_MAX_ROWS and h.shape[1] % 8 == 0
+                and out_dtype in (None, torch.bfloat16) and h.is_contiguous()):
+            return self.gemm_skinny(h, w)
         out = torch.matmul(h, w.t())
         return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
+
+    def swiglu_linear(self, h, w_gate_up):
+        """``silu(h @ Wg.T) * (h @ Wu.T)`` with ``w_gate_up`` = gate rows, then up rows."""
+        if h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_MAX_ROWS and h.shape[1] % 8 == 0:
+            return self.gemm_skinny(h, w_gate_up, swiglu=True)
+        return self.silu_mul(torch.matmul(h, w_gate_up.t()))
 
     def gemm(self, a, b, *, offsets=None, a_rows=None, scale=None, out_f32=False, rows=None):
         """The hand-written product ``C[r] = scale[r] * A[a_rows[r]] @ B[g(r)].T`` (see ``gemm_generic.hip``)."""
@@ -302,7 +339,7 @@ class HipOps:
         self._chk(router, torch.float32, (e, d), "router matrix")
         ids = torch.empty(n, top_k, dtype=torch.int32, device=h32.device)
         gates = torch.empty(n, top_k, dtype=torch.float32, device=h32.device)
-        logits = torch.empty(n, e, dtype=torch.float32, device=h32.device) if want_logits else None
+        logits = torch.empty(n, e, dtype=torch.float32, device=h32.device)
         self._call("jle_moe_route", _p(h32), _p(router), _p(ids), _p(gates), _p(logits), n, d, e, top_k)
         return (ids, gates, logits) if want_logits else (ids, gates)
 
@@ -332,11 +369,9 @@ class HipOps:
             gu = self.gemm(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate)
             act = self.silu_mul(gu)
             routed = self.gemm(act, w_down, offsets=offsets)
-        out = torch.empty(n, d, dtype=torch.float32, device=h.device)
         if shared is not None:
             self._chk(shared, h.dtype, (n, d), "shared expert output")
-        self._call("jle_moe_combine", _p(routed), _p(inv), _p(shared), _p(out), self._is_bf16(h), n, k, d)
-        return out
+        return ExpertSum(routed, inv, k, shared, n, d)
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, temperature, top_k, seeds, counters):

@@ -66,6 +66,12 @@ class ReferenceOps:
     def lm_head(self, h, w):
         return h.float() @ w.float().t()
 
+    def swiglu_linear(self, h, w_gate_up):
+        return self.silu_mul(self.linear(h, w_gate_up))
+
+    def materialize(self, delta):
+        return delta
+
     def silu_mul(self, gate_up):
         f = gate_up.shape[-1] // 2
         g, u = gate_up[..., :f].float(), gate_up[..., f:].float()

@@ -31,8 +31,7 @@ class DenseSwiGLU(FeedForward):
 
     def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
         ops = ctx.ops
-        act = ops.silu_mul(ops.linear(h, self.params["w_gate_up"]))
-        return ops.linear(act, self.params["w_down"])
+        return ops.linear(ops.swiglu_linear(h, self.params["w_gate_up"]), self.params["w_down"])
 
 
 @register_feed_forward("moe_sigmoid_shared")
@@ -70,6 +69,5 @@ class MoESigmoidShared(FeedForward):
             expert_ids, gates = forced
         shared = None
         if self.shared_inter:
-            act = ops.silu_mul(ops.linear(h, self.params["shared_gate_up"]))
-            shared = ops.linear(act, self.params["shared_down"])
+            shared = ops.linear(ops.swiglu_linear(h, self.params["shared_gate_up"]), self.params["shared_down"])
         return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"], shared)

@@ -48,7 +48,7 @@ def test_embed(ops, ref, dt):
 
 
 @pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("d", [80, 1000, 5120])
+@pytest.mark.parametrize("d", [80, 1000, 1026, 5120, 9000])
 def test_add_rmsnorm(ops, ref, dt, d):
     for delta_dt, weighted, want32 in [(None, True, False), (dt, True, True), (torch.float32, False, True)]:
         x = _rand(7, d, seed=1)
@@ -199,7 +199,8 @@ def test_attention_reading_a_page_that_was_given_back_is_not_silent(ops):
     assert torch.isnan(out).all()
 
 
-@pytest.mark.parametrize("n,d,e,k", [(50, 5120, 16, 1), (7, 80, 3, 2), (33, 96, 128, 4), (1, 64, 4, 1)])
+@pytest.mark.parametrize("n,d,e,k", [(50, 5120, 16, 1), (7, 80, 3, 2), (33, 96, 128, 4), (1, 64, 4, 1), (70, 50, 5, 2),
+                                     (300, 264, 16, 1)])
 def test_moe_route(ops, ref, n, d, e, k):
     h, w = _rand(n, d, seed=1), _rand(e, d, scale=0.05, seed=2)
     ids, gates, logits = ops.moe_route(h, w, k, want_logits=True)
@@ -226,12 +227,25 @@ def test_moe_experts(ops, ref, dt, n, d, f, e, k):
     if e > 3:
         ids[ids == 2] = 0  # an expert nobody chose
     gates = torch.rand(n, k, generator=g).to(DEV)
-    got = ops.moe_experts(h, ids, gates, wgu, wd, shared)
+    lazy = ops.moe_experts(h, ids, gates, wgu, wd, shared)  # the pieces; summed by the kernel that uses them
+    got = ops.materialize(lazy)
     want = ref.moe_experts(h, ids, gates, wgu, wd, shared)
-    assert got.dtype == torch.float32
+    assert got.dtype == torch.float32 and lazy.shape == (n, d)
     _assert_close_to_scale(got, want, dt)
-    _assert_close_to_scale(ops.moe_experts(h, ids, gates, wgu, wd, None),
+    _assert_close_to_scale(ops.materialize(ops.moe_experts(h, ids, gates, wgu, wd, None)),
                            ref.moe_experts(h, ids, gates, wgu, wd, None), dt)
+    # residual add + norm reading the pieces = the same on the summed tensor
+    x = _rand(n, d, seed=9)
+    w = _rand(d, seed=10)
+    x1, x2 = x.clone(), x.clone()
+    h1, h32 = ops.add_rmsnorm(x1, lazy, w, 1e-5, dt, True)
+    h2, h32b = ops.add_rmsnorm(x2, got, w, 1e-5, dt, True)
+    assert torch.allclose(x1, x2, rtol=1e-6, atol=1e-6) and torch.allclose(h32, h32b, rtol=1e-5, atol=1e-6)
+    x3 = x.clone()
+    ops.add_residual(x3, lazy)
+    assert torch.allclose(x3, x1, rtol=1e-6, atol=1e-6)
+    idx = torch.tensor([n - 1, 0], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.gather_rows(lazy, idx), got[idx.long()])
 
 
 def test_moe_align_is_a_stable_grouping(ops):
@@ -254,6 +268,11 @@ def test_moe_align_is_a_stable_grouping(ops):
 def test_product_kernel_and_lm_head(ops, ref, dt):
     a, b = _rand(33, 52, dt=dt, seed=1), _rand(70, 52, dt=dt, seed=2)
     _assert_close_to_scale(ops.gemm(a, b), ref.linear(a, b), dt)
+    gu = _rand(2 * 24, 52, dt=dt, seed=6)
+    for rows in (33, 100):  # few rows (weight streaming in bfloat16) and many
+        aa = _rand(rows, 52, dt=dt, seed=7)
+        _assert_close_to_scale(ops.swiglu_linear(aa, gu), ref.swiglu_linear(aa, gu), dt)
+        _assert_close_to_scale(ops.linear(aa, b), ref.linear(aa, b), dt)
     h, w = _rand(5, 80, dt=dt, seed=3), _rand(311, 80, dt=dt, seed=4)
     got = ops.lm_head(h, w)
     assert got.dtype == torch.float32 and got.shape == (5, 311)

@@ -90,7 +90,7 @@ def test_feed_forward_part_alone(model_dirs, device, name, layer):
         forced_routing: dict = None
 
     xd = x.to(device)
-    got = ff.forward(xd, xd if ff.wants_float32_input else None, Ctx(ops)).float().cpu()
+    got = ops.materialize(ff.forward(xd, xd if ff.wants_float32_input else None, Ctx(ops))).float().cpu()
     assert torch.allclose(got, want, rtol=1e-4, atol=2e-6)
     if layer in cfg["moe_layers"]:
         assert torch.equal(ff.last_routing[0].cpu().long(), idx)
