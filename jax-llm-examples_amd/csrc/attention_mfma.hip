@@ -82,6 +82,7 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
   for (int kb = (k_lo / 32) * 32; kb <= k_hi; kb += 32) {
     f32x4 st[CT][2];
     const bf16_t* vbase[2];
+    const bf16_t* krow[2];
     bool active[2];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
@@ -98,19 +99,49 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
       vbase[tt] = nullptr;
+      krow[tt] = nullptr;
       if (active[tt]) {
         const bf16_t* kbase = kv + (size_t)page * page_stride + (size_t)hk * plane;
         const int off = key0 % ps;
-        const bf16_t* krow = kbase + (size_t)(off + c16) * DH + g * 8;
+        krow[tt] = kbase + (size_t)(off + c16) * DH + g * 8;
         vbase[tt] = kbase + (size_t)Hkv * plane + off + 4 * g;  // + d * ps
+      }
+    }
+    // all loads of this step are issued first (keys, then values), so that the values arrive while the
+    // scores are worked on
+    uint4 kraw[2][KC];
 #pragma unroll
-        for (int c = 0; c < KC; ++c) {
-          const uint4 kvv = *reinterpret_cast<const uint4*>(krow + c * 32);
-          const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
+    for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-          for (int ct = 0; ct < CT; ++ct)
-            st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
-        }
+      for (int c = 0; c < KC; ++c) {
+        kraw[tt][c] = uint4{0u, 0u, 0u, 0u};
+        if (active[tt]) kraw[tt][c] = *reinterpret_cast<const uint4*>(krow[tt] + c * 32);
+      }
+    uint4 vraw[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      vraw[dt] = uint4{0u, 0u, 0u, 0u};
+      const size_t drow = (size_t)(dt * 16 + c16) * ps;
+      if (active[0]) {
+        const uint2 t0 = *reinterpret_cast<const uint2*>(vbase[0] + drow);
+        vraw[dt].x = t0.x;
+        vraw[dt].y = t0.y;
+      }
+      if (active[1]) {
+        const uint2 t1 = *reinterpret_cast<const uint2*>(vbase[1] + drow);
+        vraw[dt].z = t1.x;
+        vraw[dt].w = t1.y;
+      }
+    }
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      if (!active[tt]) continue;
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, kraw[tt][c]);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+          st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
       }
     }
     // mask, running max and sum per column
@@ -169,18 +200,11 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
     }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      uint4 vv = {0u, 0u, 0u, 0u};
-      const size_t drow = (size_t)(dt * 16 + c16) * ps;
-      if (active[0]) {
-        const uint2 t0 = *reinterpret_cast<const uint2*>(vbase[0] + drow);
-        vv.x = t0.x & keep[0][0];
-        vv.y = t0.y & keep[0][1];
-      }
-      if (active[1]) {
-        const uint2 t1 = *reinterpret_cast<const uint2*>(vbase[1] + drow);
-        vv.z = t1.x & keep[1][0];
-        vv.w = t1.y & keep[1][1];
-      }
+      uint4 vv = vraw[dt];
+      vv.x &= keep[0][0];
+      vv.y &= keep[0][1];
+      vv.z &= keep[1][0];
+      vv.w &= keep[1][1];
       const bf16x8 a = __builtin_bit_cast(bf16x8, vv);
 #pragma unroll
       for (int ct = 0; ct < CT; ++ct)

@@ -34,14 +34,13 @@ __device__ __forceinline__ void store_out<float>(float* p, float v) { *p = v; }
 template <>
 __device__ __forceinline__ void store_out<bf16_t>(bf16_t* p, float v) { *p = float_to_bf16(v); }
 
-constexpr int kUnroll = 4;
-
-template <int MT, bool SWIGLU, typename OutT>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
+template <int MT, bool SWIGLU, typename OutT, int WAVES, int kUnroll, int RT = 2>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                           OutT* __restrict__ Y, const int* __restrict__ offsets,
                                                           const int* __restrict__ a_rows,
                                                           const float* __restrict__ scale, int M, int Nout, int K) {
-  __shared__ float red[4][2 * MT * 4][64];
+  static_assert(RT == 2 || !SWIGLU, "the fused activation needs the gate tile and the up tile");
+  __shared__ float red[WAVES][RT * MT * 4][64];
   const int e = blockIdx.z;
   int row_lo = 0, row_hi = M;
   if (offsets != nullptr) {
@@ -54,7 +53,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
   const int r = lane & 15, g = lane >> 4;
   const bf16_t* We = W + (size_t)e * Nout * K;
   const int half = Nout >> 1;
-  const int base = SWIGLU ? blockIdx.x * 16 : blockIdx.x * 32;  // first output column of the block
+  const int base = SWIGLU ? blockIdx.x * 16 : blockIdx.x * (16 * RT);  // first output column of the block
   int ra0, ra1;  // the weight rows this lane reads
   if (SWIGLU) {
     ra0 = min(base + r, half - 1);
@@ -81,14 +80,14 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
     acc1[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int nkb = (K + 31) >> 5;
-  for (int kb0 = wave; kb0 < nkb; kb0 += 4 * kUnroll) {
+  for (int kb0 = wave; kb0 < nkb; kb0 += WAVES * kUnroll) {
     bf16x8 A0[kUnroll], A1[kUnroll], B[kUnroll][MT];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      const int kb = kb0 + 4 * u;
+      const int kb = kb0 + WAVES * u;
       const bool ok = kb < nkb && (kb * 32 + g * 8) < K;  // K is a multiple of 8
       A0[u] = ok ? load8(a0 + kb * 32) : zero8();
-      A1[u] = ok ? load8(a1 + kb * 32) : zero8();
+      if (RT == 2) A1[u] = ok ? load8(a1 + kb * 32) : zero8();
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) B[u][mt] = (ok && xv[mt]) ? load8(xb[mt] + kb * 32) : zero8();
     }
@@ -97,7 +96,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         acc0[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A0[u], B[u][mt], acc0[mt], 0, 0, 0);
-        acc1[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[u], B[u][mt], acc1[mt], 0, 0, 0);
+        if (RT == 2) acc1[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[u], B[u][mt], acc1[mt], 0, 0, 0);
       }
     }
   }
@@ -106,59 +105,98 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       red[wave][(0 * MT + mt) * 4 + i][lane] = acc0[mt][i];
-      red[wave][(1 * MT + mt) * 4 + i][lane] = acc1[mt][i];
+      if (RT == 2) red[wave][(1 * MT + mt) * 4 + i][lane] = acc1[mt][i];
     }
   }
   __syncthreads();
-  // wavefront w finishes element i = w of every tile: D[row 4 * g + i of the tile][token r]
-  const int i = wave;
-  const int m = g * 4 + i;
+  // wavefront w < 4 finishes element i = w of every tile: D[row 4 * g + i of the tile][token r]
+  // (a block of one wavefront finishes all four)
+  if (wave >= 4) return;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    float v0 = 0.f, v1 = 0.f;
+  for (int ii = 0; ii < 4; ++ii) {
+    if (WAVES > 1 && ii != wave) continue;
+    const int i = ii;
+    const int m = g * 4 + i;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      v0 += red[w][(0 * MT + mt) * 4 + i][lane];
-      v1 += red[w][(1 * MT + mt) * 4 + i][lane];
-    }
-    const int t = tok0 + mt * 16 + r;
-    if (t >= row_hi) continue;
-    const float sc = scale != nullptr ? scale[t] : 1.f;
-    if (SWIGLU) {
-      const int f = base + m;
-      if (f < half) {
-        const float gate = v0 * sc, up = v1 * sc;
-        store_out<OutT>(Y + (size_t)t * half + f, gate / (1.0f + expf(-gate)) * up);
+    for (int mt = 0; mt < MT; ++mt) {
+      float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) {
+        v0 += red[w][(0 * MT + mt) * 4 + i][lane];
+        if (RT == 2) v1 += red[w][(1 * MT + mt) * 4 + i][lane];
       }
-    } else {
-      const int c0 = base + m, c1 = base + 16 + m;
-      if (c0 < Nout) store_out<OutT>(Y + (size_t)t * Nout + c0, v0 * sc);
-      if (c1 < Nout) store_out<OutT>(Y + (size_t)t * Nout + c1, v1 * sc);
+      const int t = tok0 + mt * 16 + r;
+      if (t >= row_hi) continue;
+      const float sc = scale != nullptr ? scale[t] : 1.f;
+      if (SWIGLU) {
+        const int f = base + m;
+        if (f < half) {
+          const float gate = v0 * sc, up = v1 * sc;
+          store_out<OutT>(Y + (size_t)t * half + f, gate / (1.0f + expf(-gate)) * up);
+        }
+      } else {
+        const int c0 = base + m, c1 = base + 16 + m;
+        if (c0 < Nout) store_out<OutT>(Y + (size_t)t * Nout + c0, v0 * sc);
+        if (RT == 2 && c1 < Nout) store_out<OutT>(Y + (size_t)t * Nout + c1, v1 * sc);
+      }
     }
   }
 }
 
 // X [*, K] bf16, W [G, Nout, K] bf16, Y [M, Nout] (or [M, Nout / 2] with swiglu) bf16 or float32.
-// max_rows: the most rows any group can have (M if unknown).
+// max_rows: the most rows any group can have (M if unknown).  variant: 0 = chosen from the
+// sizes; else waves * 16 + unroll (for tuning).
+// variant = row tiles * 256 + wavefronts * 16 + unroll
+template <int MT, bool SW, typename OT>
+static int launch_skinny(int xrows, int ytiles, int G, hipStream_t s, int variant, const void* X, const void* W,
+                         void* Y, const int* offsets, const int* a_rows, const float* scale, int M, int Nout, int K) {
+#define LAUNCH(RT, WV, UN)                                                                                       \
+  do {                                                                                                           \
+    dim3 g((xrows + 16 * (SW ? 1 : RT) - 1) / (16 * (SW ? 1 : RT)), ytiles, G);                                  \
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, SW, OT, WV, UN, (SW ? 2 : RT)>), g, dim3(WV * 64), 0, s,          \
+                       (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, offsets, a_rows, scale, M, Nout, K);          \
+    return 0;                                                                                                    \
+  } while (0)
+  switch (variant) {
+    case 2 * 256 + 4 * 16 + 4: LAUNCH(2, 4, 4);
+    case 2 * 256 + 4 * 16 + 8: LAUNCH(2, 4, 8);
+    case 2 * 256 + 2 * 16 + 8: LAUNCH(2, 2, 8);
+    case 2 * 256 + 1 * 16 + 8: LAUNCH(2, 1, 8);
+    case 1 * 256 + 8 * 16 + 4: LAUNCH(1, 8, 4);
+    case 1 * 256 + 4 * 16 + 8: LAUNCH(1, 4, 8);
+    case 1 * 256 + 2 * 16 + 8: LAUNCH(1, 2, 8);
+    case 1 * 256 + 1 * 16 + 8: LAUNCH(1, 1, 8);
+  }
+#undef LAUNCH
+  return JLE_BAD_ARG;
+}
+
+// X [*, K] bf16, W [G, Nout, K] bf16, Y [M, Nout] (or [M, Nout / 2] with swiglu) bf16 or float32.
+// max_rows: the most rows any group can have (M if unknown).  variant: 0 = chosen from the sizes.
 JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* offsets, const int* a_rows,
                             const float* scale, int swiglu, int out_f32, int M, int Nout, int K, int G, int max_rows,
-                            hipStream_t s) {
+                            int variant, hipStream_t s) {
   if (M <= 0 || Nout <= 0) return 0;
   if (K <= 0 || K % 8 || G < 1 || G > 65535 || (swiglu && Nout % 2)) return JLE_BAD_ARG;
   if (max_rows <= 0 || max_rows > M) max_rows = M;
   const int mt = (offsets == nullptr && max_rows > 32) ? 4 : (offsets == nullptr && max_rows > 16) ? 2 : 1;
   const int ytiles = (max_rows + 16 * mt - 1) / (16 * mt);
   if (ytiles > 65535) return JLE_BAD_ARG;
-  const int xtiles = swiglu ? (Nout / 2 + 15) / 16 : (Nout + 31) / 32;
-  dim3 g(xtiles, ytiles, G), b(256);
-#define LAUNCH(MT, SW, OT)                                                                                     \
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, SW, OT>), g, b, 0, s, (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, \
-                     offsets, a_rows, scale, M, Nout, K)
-#define PICK(SW, OT)              \
-  do {                            \
-    if (mt == 1) LAUNCH(1, SW, OT); \
-    else if (mt == 2) LAUNCH(2, SW, OT); \
-    else LAUNCH(4, SW, OT);       \
+  const int xrows = swiglu ? Nout / 2 : Nout;  // output columns to cover
+  if (variant == 0) {
+    // measured on MI355X at 1 to 64 rows (Scout's expert, attention and head shapes)
+    const long long groups = offsets != nullptr ? (G < M ? G : M) : 1;
+    const long long pair_tiles = (long long)((xrows + (swiglu ? 15 : 31)) / (swiglu ? 16 : 32)) * groups;
+    if (swiglu) variant = 2 * 256 + 4 * 16 + 8;
+    else if (pair_tiles >= 4096) variant = 2 * 256 + 4 * 16 + 8;  // very many rows of W (the output head)
+    else variant = 1 * 256 + 8 * 16 + 4;  // one row tile per block, 8 wavefronts split K: more blocks in flight
+  }
+  int rc;
+#define PICK(SW, OT)                                                                                             \
+  do {                                                                                                           \
+    if (mt == 1) rc = launch_skinny<1, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K);      \
+    else if (mt == 2) rc = launch_skinny<2, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K); \
+    else rc = launch_skinny<4, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K);              \
   } while (0)
   if (swiglu) {
     if (out_f32) PICK(true, float); else PICK(true, bf16_t);
@@ -166,7 +204,7 @@ JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* of
     if (out_f32) PICK(false, float); else PICK(false, bf16_t);
   }
 #undef PICK
-#undef LAUNCH
+  if (rc != 0) return rc;
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -33,7 +33,8 @@ _SIGNATURES = {
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
     "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
     "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
-    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
 
@@ -175,17 +176,13 @@ class HipOps:
 
     # ------------------------------------------------------------------ matrix products
     def linear(self, h, w, out_dtype=None):
-        """``h @ w.T``.  Few bfloat16 rows: the weight-streaming MFMA kernel; otherwise the BLAS library
-        (float32: true float32)."""
-        if (h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_MAX_ROWS and h.shape[1] % 8 == 0
-                and out_dtype in (None, torch.bfloat16) and h.is_contiguous()):
-            return self.gemm_skinny(h, w)
+        """``h @ w.T`` through the BLAS library (float32: true float32)."""
         out = torch.matmul(h, w.t())
         return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
 
     def swiglu_linear(self, h, w_gate_up):
         """``silu(h @ Wg.T) * (h @ Wu.T)`` with ``w_gate_up`` = gate rows, then up rows."""
-        if h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_MAX_ROWS and h.shape[1] % 8 == 0:
+        if h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_DENSE_ROWS and h.shape[1] % 8 == 0:
             return self.gemm_skinny(h, w_gate_up, swiglu=True)
         return self.silu_mul(torch.matmul(h, w_gate_up.t()))
 
@@ -205,8 +202,10 @@ class HipOps:
         return out
 
     SKINNY_MAX_ROWS = 64  # up to here a product is a stream of the weights: the MFMA weight-streaming kernel
+    SKINNY_DENSE_ROWS = 16  # the fused gate|up projection of a dense feed-forward: beyond this the BLAS library
 
-    def gemm_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None):
+    def gemm_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
+                    variant=0):
         """bfloat16 weight-streaming product on MFMA for few rows (see ``gemm_skinny.hip``); with ``swiglu`` the
         result is ``silu(gate) * up`` of the two halves of ``b``'s rows."""
         if b.dim() == 2:
@@ -222,14 +221,34 @@ class HipOps:
         out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
                           device=a.device)
         self._call("jle_gemm_skinny", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
-                   int(out_f32), m, nout, k, g, m)
+                   int(out_f32), m, nout, k, g, m, variant)
+        return out
+
+    def gemm_grouped(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None):
+        """bfloat16 product on MFMA for many rows, grouped by ``offsets`` (see ``gemm_grouped.hip``)."""
+        if b.dim() == 2:
+            b = b.unsqueeze(0)
+        g, nout, k = b.shape
+        m = rows if rows is not None else (a_rows.numel() if a_rows is not None else a.shape[0])
+        self._chk(a, torch.bfloat16, None, "A")
+        self._chk(b, torch.bfloat16, None, "B")
+        if a.shape[1] != k:
+            raise KernelError(f"inner sizes differ: A {tuple(a.shape)}, B {tuple(b.shape)}")
+        if k % 8:
+            raise KernelError(f"the MFMA product needs an inner size that is a multiple of 8, got {k}")
+        out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
+                          device=a.device)
+        self._call("jle_gemm_grouped", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
+                   int(out_f32), m, nout, k, g)
         return out
 
     def lm_head(self, h, w):
         if h.dtype == torch.float32:
             return torch.matmul(h, w.t())
-        if h.shape[0] <= self.SKINNY_MAX_ROWS and h.shape[1] % 8 == 0:
-            return self.gemm_skinny(h, w, out_f32=True)
+        if h.shape[1] % 8 == 0:
+            if h.shape[0] <= self.SKINNY_MAX_ROWS:
+                return self.gemm_skinny(h, w, out_f32=True)
+            return self.gemm_grouped(h, w, out_f32=True)
         return self.gemm(h, w, out_f32=True)
 
     def silu_mul(self, gate_up):
@@ -362,9 +381,13 @@ class HipOps:
         e, f2, _ = w_gate_up.shape
         k = expert_ids.shape[1]
         offsets, sorted_token, sorted_gate, inv = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e)
-        if h.dtype == torch.bfloat16 and n * k <= 2 * self.SKINNY_MAX_ROWS and d % 8 == 0 and (f2 // 2) % 8 == 0:
+        mfma = h.dtype == torch.bfloat16 and d % 8 == 0 and (f2 // 2) % 8 == 0
+        if mfma and n * k <= 2 * self.SKINNY_MAX_ROWS:  # few rows: the cost is streaming the chosen experts' weights
             act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True)
             routed = self.gemm_skinny(act, w_down, offsets=offsets)
+        elif mfma:
+            act = self.gemm_grouped(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True)
+            routed = self.gemm_grouped(act, w_down, offsets=offsets)
         else:
             gu = self.gemm(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate)
             act = self.silu_mul(gu)

@@ -355,3 +355,35 @@ def test_weight_streaming_product_grouped_with_swiglu(ops, ref, n, d, f, e, k):
     assert float((act.float() - want).abs().max() / want.abs().max()) <= 5e-3
     plain = ops.gemm_skinny(h, wgu, offsets=off, a_rows=tok, scale=gate, out_f32=True)
     assert float((plain - gu).abs().max() / gu.abs().max()) <= 2e-5
+
+
+@pytest.mark.parametrize("n,d,f,e,k", [(300, 128, 48, 16, 1), (700, 264, 72, 3, 2), (2048, 512, 256, 16, 1),
+                                       (150, 64, 40, 128, 1)])
+def test_grouped_product_for_many_rows(ops, ref, n, d, f, e, k):
+    dt = torch.bfloat16
+    h = _rand(n, d, dt=dt, seed=1)
+    wgu = _rand(e, 2 * f, d, dt=dt, scale=0.1, seed=2)
+    wd = _rand(e, d, f, dt=dt, scale=0.1, seed=3)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(n)]).to(torch.int32).to(DEV)
+    if n == 300:
+        ids[:200] = 3  # one expert with more rows than one block, others with none
+    gates = torch.rand(n, k, generator=g).to(DEV)
+    off, tok, gate, inv = ops.moe_align(ids, gates, e)
+    act = ops.gemm_grouped(h, wgu, offsets=off, a_rows=tok, scale=gate, swiglu=True)
+    gu = ops.gemm(h, wgu, offsets=off, a_rows=tok, scale=gate, out_f32=True)  # the general kernel, float32 result
+    want = torch.nn.functional.silu(gu[:, :f]) * gu[:, f:]
+    assert act.shape == (n * k, f)
+    assert float((act.float() - want).abs().max() / want.abs().max()) <= 5e-3
+    plain = ops.gemm_grouped(h, wgu, offsets=off, a_rows=tok, scale=gate, out_f32=True)
+    assert float((plain - gu).abs().max() / gu.abs().max()) <= 2e-5
+    down = ops.gemm_grouped(act, wd, offsets=off)
+    want_d = ops.gemm(act, wd, offsets=off, out_f32=True)
+    assert float((down.float() - want_d).abs().max() / want_d.abs().max()) <= 5e-3
+    # the whole expert layer at this size takes the same path
+    _assert_close_to_scale(ops.materialize(ops.moe_experts(h, ids, gates, wgu, wd, None)),
+                           ref.moe_experts(h, ids, gates, wgu, wd, None), dt)
+    dense = ops.gemm_grouped(h, wgu[0], out_f32=True)  # one group, no offsets
+    assert float((dense - h.float() @ wgu[0].float().t()).abs().max() / dense.abs().max()) <= 2e-5
+    head = ops.lm_head(h[:100, :], _rand(311, d, dt=dt, seed=7))
+    assert head.dtype == torch.float32 and head.shape == (100, 311)
