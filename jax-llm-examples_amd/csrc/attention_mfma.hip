@@ -79,11 +79,12 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
     for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int kb = (k_lo / 32) * 32; kb <= k_hi; kb += 32) {
-    f32x4 st[CT][2];
-    const bf16_t* vbase[2];
-    const bf16_t* krow[2];
-    bool active[2];
+  // The keys of a step are asked for one step ahead (they are in registers when the step begins); its
+  // values are asked for at its beginning and arrive while the scores are worked on.
+  uint4 kraw[2][KC];
+  const bf16_t* vbase[2];
+  bool active[2];
+  auto locate_and_load_keys = [&](int kb) {
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
       const int key0 = kb + 16 * tt;
@@ -96,46 +97,46 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
           active[tt] = false;
         }
       }
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
       vbase[tt] = nullptr;
-      krow[tt] = nullptr;
+#pragma unroll
+      for (int c = 0; c < KC; ++c) kraw[tt][c] = uint4{0u, 0u, 0u, 0u};
       if (active[tt]) {
         const bf16_t* kbase = kv + (size_t)page * page_stride + (size_t)hk * plane;
         const int off = key0 % ps;
-        krow[tt] = kbase + (size_t)(off + c16) * DH + g * 8;
+        const bf16_t* krow = kbase + (size_t)(off + c16) * DH + g * 8;
         vbase[tt] = kbase + (size_t)Hkv * plane + off + 4 * g;  // + d * ps
+#pragma unroll
+        for (int c = 0; c < KC; ++c) kraw[tt][c] = *reinterpret_cast<const uint4*>(krow + c * 32);
       }
     }
-    // all loads of this step are issued first (keys, then values), so that the values arrive while the
-    // scores are worked on
-    uint4 kraw[2][KC];
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int c = 0; c < KC; ++c) {
-        kraw[tt][c] = uint4{0u, 0u, 0u, 0u};
-        if (active[tt]) kraw[tt][c] = *reinterpret_cast<const uint4*>(krow[tt] + c * 32);
-      }
+  };
+  const int kb_first = (k_lo / 32) * 32;
+  if (kb_first <= k_hi) locate_and_load_keys(kb_first);
+  for (int kb = kb_first; kb <= k_hi; kb += 32) {
+    f32x4 st[CT][2];
+    const bool act0 = active[0], act1 = active[1];
+    // this step's values
     uint4 vraw[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       vraw[dt] = uint4{0u, 0u, 0u, 0u};
       const size_t drow = (size_t)(dt * 16 + c16) * ps;
-      if (active[0]) {
+      if (act0) {
         const uint2 t0 = *reinterpret_cast<const uint2*>(vbase[0] + drow);
         vraw[dt].x = t0.x;
         vraw[dt].y = t0.y;
       }
-      if (active[1]) {
+      if (act1) {
         const uint2 t1 = *reinterpret_cast<const uint2*>(vbase[1] + drow);
         vraw[dt].z = t1.x;
         vraw[dt].w = t1.y;
       }
     }
+    // scores from the keys that are already here
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      if (!active[tt]) continue;
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < KC; ++c) {
         const bf16x8 a = __builtin_bit_cast(bf16x8, kraw[tt][c]);
@@ -144,6 +145,8 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
           st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
       }
     }
+    // the next step's keys (overwrites kraw, vbase and active: this step keeps act0 / act1 and vraw)
+    if (kb + 32 <= k_hi) locate_and_load_keys(kb + 32);
     // mask, running max and sum per column
     bf16x8 pb[CT];
 #pragma unroll
@@ -155,7 +158,7 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = kb + 16 * tt + 4 * g + i;
-          const bool ok = active[tt] && key >= col[ct].lo && key <= col[ct].hi;
+          const bool ok = (tt == 0 ? act0 : act1) && key >= col[ct].lo && key <= col[ct].hi;
           const float v = ok ? st[ct][tt][i] * scale_log2 : -INFINITY;
           s[tt * 4 + i] = v;
           mx = fmaxf(mx, v);
@@ -225,7 +228,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (item >= num_tiles * Hq) return;
-  const int tile = item / Hq, h = item - tile * Hq;
+  // the last tiles of a segment have the most keys: they are started first
+  const int tile = num_tiles - 1 - item / Hq, h = item % Hq;
   const int n0 = tiles[2 * tile], nt = tiles[2 * tile + 1];
   const int hk = h / (Hq / Hkv);
   const int c16 = lane & 15, g = lane >> 4;

@@ -109,23 +109,25 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
     const int src = xok[i] ? (a_rows != nullptr ? a_rows[tok] : tok) : 0;
     xsrc[i] = X + (size_t)src * K + kc;
   }
-  uint4 wreg[4], xreg[4];
-  auto load_tile = [&](int k0) {
+  // two register sets: the tile two steps ahead is on its way while the tile one step ahead waits to be
+  // written to shared memory, so a load has two steps of matrix work to arrive
+  uint4 wreg[2][4], xreg[2][4];
+  auto load_tile = [&](int set, int k0) {
     const bool kok = k0 + kc < K;  // K is a multiple of 8
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      wreg[i] = uint4{0u, 0u, 0u, 0u};
-      xreg[i] = uint4{0u, 0u, 0u, 0u};
-      if (kok) wreg[i] = *reinterpret_cast<const uint4*>(wsrc[i] + k0);
-      if (kok && xok[i]) xreg[i] = *reinterpret_cast<const uint4*>(xsrc[i] + k0);
+      wreg[set][i] = uint4{0u, 0u, 0u, 0u};
+      xreg[set][i] = uint4{0u, 0u, 0u, 0u};
+      if (kok) wreg[set][i] = *reinterpret_cast<const uint4*>(wsrc[i] + k0);
+      if (kok && xok[i]) xreg[set][i] = *reinterpret_cast<const uint4*>(xsrc[i] + k0);
     }
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](int set, int buf) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int rr = (t >> 3) + 32 * i;
-      *reinterpret_cast<uint4*>(&sW[buf][rr * PITCH + kc]) = wreg[i];
-      *reinterpret_cast<uint4*>(&sX[buf][rr * PITCH + kc]) = xreg[i];
+      *reinterpret_cast<uint4*>(&sW[buf][rr * PITCH + kc]) = wreg[set][i];
+      *reinterpret_cast<uint4*>(&sX[buf][rr * PITCH + kc]) = xreg[set][i];
     }
   };
 
@@ -138,33 +140,43 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
   const bool wave_has_rows = row0 + wm * 64 < row_end;
 
   const int nk = (K + BK - 1) / BK;
-  load_tile(0);
-  store_tile(0);
+  load_tile(0, 0);
+  store_tile(0, 0);
+  if (nk > 1) load_tile(1, BK);
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) load_tile((kt + 1) * BK);
-    if (wave_has_rows) {
+  // the loop is unrolled by two so that the register sets are named at compile time
+  auto compute = [&](int buf) {
+    if (!wave_has_rows) return;
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        bf16x8 a[4], b[4];
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16x8 a[4], b[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint4 v = *reinterpret_cast<const uint4*>(&sW[buf][(wn * 64 + j * 16 + c16) * PITCH + ks * 32 + g * 8]);
-          a[j] = __builtin_bit_cast(bf16x8, v);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint4 v = *reinterpret_cast<const uint4*>(&sX[buf][(wm * 64 + i * 16 + c16) * PITCH + ks * 32 + g * 8]);
-          b[i] = __builtin_bit_cast(bf16x8, v);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[i], acc[j][i], 0, 0, 0);
+      for (int j = 0; j < 4; ++j) {
+        const uint4 v = *reinterpret_cast<const uint4*>(&sW[buf][(wn * 64 + j * 16 + c16) * PITCH + ks * 32 + g * 8]);
+        a[j] = __builtin_bit_cast(bf16x8, v);
       }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint4 v = *reinterpret_cast<const uint4*>(&sX[buf][(wm * 64 + i * 16 + c16) * PITCH + ks * 32 + g * 8]);
+        b[i] = __builtin_bit_cast(bf16x8, v);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[i], acc[j][i], 0, 0, 0);
     }
-    if (kt + 1 < nk) store_tile(buf ^ 1);
+  };
+  for (int kt = 0; kt < nk; kt += 2) {
+    // even step: tile kt is in buffer 0, tile kt + 1 in register set 1
+    if (kt + 2 < nk) load_tile(0, (kt + 2) * BK);
+    compute(0);
+    if (kt + 1 < nk) store_tile(1, 1);
+    __syncthreads();
+    if (kt + 1 >= nk) break;
+    // odd step: tile kt + 1 is in buffer 1, tile kt + 2 in register set 0
+    if (kt + 3 < nk) load_tile(1, (kt + 3) * BK);
+    compute(1);
+    if (kt + 2 < nk) store_tile(0, 0);
     __syncthreads();
   }
   if (!wave_has_rows) return;
