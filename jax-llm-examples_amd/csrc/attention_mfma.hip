@@ -20,9 +20,11 @@
 // as they are.  The A operand of that product then reads, for element d, keys 4g..4g+3 of each
 // tile: 8 contiguous bytes of the transposed value page.
 //
-// Decode splits a token's keys into ranges of kSplit absolute positions; each range is one
-// work item and leaves (max, sum, unnormalised O); a second kernel merges them in order.  Which
-// ranges and tiles a query visits depends only on its position and the retention rule.
+// Decode splits a token's keys into ranges of `split` absolute positions (a multiple of 32 that the
+// caller picks from the size of the batch, so that few long requests still fill the GPU); each
+// range is one work item and leaves (max, sum, unnormalised O); a second kernel merges them in
+// order.  Which ranges and tiles a query visits depends only on its position, the retention rule
+// and `split`.
 #include "common.h"
 
 using namespace jle;
@@ -30,7 +32,6 @@ using namespace jle;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr int kSplit = 256;  // keys per decode work item
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ int first_key(int mode, int param, int pos) {
@@ -275,8 +276,8 @@ template <int DH, int CT>
 __global__ __launch_bounds__(256) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, float* __restrict__ ws_ml, float* __restrict__ ws_o,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
-    int table_width, const int* __restrict__ dec_tokens, int num_dec, int max_splits, int ret_mode, int ret_param,
-    float scale_log2, int Hq, int Hkv, int ps) {
+    int table_width, const int* __restrict__ dec_tokens, int num_dec, int max_splits, int kSplit, int ret_mode,
+    int ret_param, float scale_log2, int Hq, int Hkv, int ps) {
   const int lane = threadIdx.x & 63;
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (item >= num_dec * Hkv * max_splits) return;
@@ -325,8 +326,8 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
 // Merges a decode token's key ranges, in order.  One block of DH threads per (decode token, head).
 __global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
                                               bf16_t* __restrict__ out, const int* __restrict__ positions,
-                                              const int* __restrict__ dec_tokens, int max_splits, int ret_mode,
-                                              int ret_param, int Hq, int Hkv, int DH, int cols) {
+                                              const int* __restrict__ dec_tokens, int max_splits, int kSplit,
+                                              int ret_mode, int ret_param, int Hq, int Hkv, int DH, int cols) {
   const int d = blockIdx.x / Hq, h = blockIdx.x % Hq;
   const int n = dec_tokens[d];
   const int pos = positions[n];
@@ -389,10 +390,11 @@ JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, cons
 // ws_ml needs num_dec * Hkv * max_splits * cols * 2 floats, ws_o that many * dh / 2, cols = 16 or 32.
 JLE_API int jle_attention_decode(const void* q, const void* kv, void* out, float* ws_ml, float* ws_o,
                                  const int* positions, const int* token_segment, const int* block_table,
-                                 int table_width, const int* dec_tokens, int num_dec, int max_splits, int ret_mode,
-                                 int ret_param, float scale, int Hq, int Hkv, int dh, int ps, hipStream_t s) {
+                                 int table_width, const int* dec_tokens, int num_dec, int max_splits, int split,
+                                 int ret_mode, int ret_param, float scale, int Hq, int Hkv, int dh, int ps,
+                                 hipStream_t s) {
   if (num_dec <= 0) return 0;
-  if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps) || max_splits < 1) return JLE_BAD_ARG;
+  if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps) || max_splits < 1 || split < 32 || split % 32) return JLE_BAD_ARG;
   if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
   const int G = Hq / Hkv;
   if (G > 32) return JLE_BAD_ARG;
@@ -403,7 +405,7 @@ JLE_API int jle_attention_decode(const void* q, const void* kv, void* out, float
 #define LAUNCH(DH, CT)                                                                                              \
   hipLaunchKernelGGL((attention_decode_kernel<DH, CT>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv, ws_ml,     \
                      ws_o, positions, token_segment, block_table, table_width, dec_tokens, num_dec, max_splits,     \
-                     ret_mode, ret_param, sl, Hq, Hkv, ps)
+                     split, ret_mode, ret_param, sl, Hq, Hkv, ps)
 #define PICK(DH)          \
   do {                    \
     if (ct == 1) LAUNCH(DH, 1); \
@@ -420,7 +422,7 @@ JLE_API int jle_attention_decode(const void* q, const void* kv, void* out, float
 #undef LAUNCH
   JLE_LAUNCH_CHECK();
   hipLaunchKernelGGL(attention_decode_merge_kernel, dim3(num_dec * Hq), dim3(dh <= 64 ? 64 : 128), 0, s, ws_ml, ws_o,
-                     (bf16_t*)out, positions, dec_tokens, max_splits, ret_mode, ret_param, Hq, Hkv, dh, 16 * ct);
+                     (bf16_t*)out, positions, dec_tokens, max_splits, split, ret_mode, ret_param, Hq, Hkv, dh, 16 * ct);
   JLE_LAUNCH_CHECK();
   return 0;
 }

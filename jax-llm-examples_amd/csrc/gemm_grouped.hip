@@ -5,11 +5,11 @@
 //
 // Rows t are sorted by group: offsets[g] .. offsets[g + 1] use W[g] (offsets == nullptr: one
 // group).  A block computes 128 rows of X against 128 rows of W (SWIGLU: 64 gate rows and their
-// 64 up rows), K in steps of 64 through shared memory, double buffered: while the matrix cores
-// work on one step, the next is on its way from memory into registers.  4 wavefronts, each
-// 64 x 64 of the result as 4 x 4 tiles of 16x16x32.  The rows of W are the A operand and the
-// rows of X the B operand, both read from shared memory with 16-byte reads; a row pitch of 72
-// elements keeps those reads free of bank conflicts.
+// 64 up rows), K in steps of BK through shared memory, double buffered, and the tile two steps
+// ahead is already on its way from memory into registers while the matrix cores work.  4
+// wavefronts, each 64 x 64 of the result as 4 x 4 tiles of 16x16x32.  The rows of W are the A
+// operand and the rows of X the B operand, both read from shared memory with 16-byte reads; the
+// row pitch (BK + 8 elements) keeps those reads free of bank conflicts.
 #include "common.h"
 
 using namespace jle;
@@ -20,8 +20,10 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 namespace {
 constexpr int BM = 128;    // rows of X per block
 constexpr int BN = 128;    // rows of W per block
-constexpr int BK = 64;     // K per step
-constexpr int PITCH = 72;  // elements between rows in shared memory (64 + 8)
+constexpr int BK = 64;     // K per step (32 was measured slower: more barriers per product)
+constexpr int PITCH = 72;  // elements between rows in shared memory (64 + 8): 16-byte reads of 16 rows hit all banks
+constexpr int CPT = BM * BK / 8 / 256;  // 16-byte chunks per thread and matrix
+constexpr int CPR = BK / 8;             // chunks per row
 
 template <typename OutT>
 __device__ __forceinline__ void store4(OutT* p, float a, float b, float c, float d, bool vec);
@@ -88,14 +90,14 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
   const int c16 = lane & 15, g = lane >> 4;
   const int wn = wave & 1, wm = wave >> 1;
 
-  // loader: 4 chunks of 16 bytes per matrix and thread; chunk c = t + 256 i: row c / 8, k offset (c % 8) * 8
-  const bf16_t* wsrc[4];
-  const bf16_t* xsrc[4];
-  bool xok[4];
-  const int kc = (t & 7) * 8;
+  // loader: CPT chunks of 16 bytes per matrix and thread; chunk c = t + 256 i: row c / CPR, k offset (c % CPR) * 8
+  const bf16_t* wsrc[CPT];
+  const bf16_t* xsrc[CPT];
+  bool xok[CPT];
+  const int kc = (t % CPR) * 8;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int rr = (t >> 3) + 32 * i;
+  for (int i = 0; i < CPT; ++i) {
+    const int rr = t / CPR + (256 / CPR) * i;
     int wrow;
     if (SWIGLU) {  // shared row rr: wavefront half rr / 64; within it 32 gate rows, then their 32 up rows
       const int j = rr & 63, f = n0 + (rr >> 6) * 32 + (j & 31);
@@ -111,11 +113,11 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
   }
   // two register sets: the tile two steps ahead is on its way while the tile one step ahead waits to be
   // written to shared memory, so a load has two steps of matrix work to arrive
-  uint4 wreg[2][4], xreg[2][4];
+  uint4 wreg[2][CPT], xreg[2][CPT];
   auto load_tile = [&](int set, int k0) {
     const bool kok = k0 + kc < K;  // K is a multiple of 8
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < CPT; ++i) {
       wreg[set][i] = uint4{0u, 0u, 0u, 0u};
       xreg[set][i] = uint4{0u, 0u, 0u, 0u};
       if (kok) wreg[set][i] = *reinterpret_cast<const uint4*>(wsrc[i] + k0);
@@ -124,8 +126,8 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
   };
   auto store_tile = [&](int set, int buf) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int rr = (t >> 3) + 32 * i;
+    for (int i = 0; i < CPT; ++i) {
+      const int rr = t / CPR + (256 / CPR) * i;
       *reinterpret_cast<uint4*>(&sW[buf][rr * PITCH + kc]) = wreg[set][i];
       *reinterpret_cast<uint4*>(&sX[buf][rr * PITCH + kc]) = xreg[set][i];
     }
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
   auto compute = [&](int buf) {
     if (!wave_has_rows) return;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < BK / 32; ++ks) {
       bf16x8 a[4], b[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {

@@ -97,7 +97,7 @@ JLE_API int jle_moe_route(const float* h, const float* w, int* ids, float* gates
   if (N <= 0) return 0;
   if (k < 1 || k > kMaxTopK || k > E || E > 4096 || logits == nullptr) return JLE_BAD_ARG;
   const bool vec = D % 4 == 0 && (((uintptr_t)h | (uintptr_t)w) & 15) == 0;
-  const bool many = N >= 64;
+  const bool many = N >= 512;  // fewer rows: a block per token keeps more blocks in flight
   dim3 g(many ? (N + 7) / 8 : N, (E + 3) / 4), b(256);
   if (many) {
     if (vec) hipLaunchKernelGGL((moe_logits_kernel<8, true>), g, b, 0, s, h, w, logits, N, D, E);

@@ -32,7 +32,8 @@ _SIGNATURES = {
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
     "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
-    "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
+    "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i,
+                             _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
@@ -280,27 +281,33 @@ class HipOps:
                    n, hq, hk, dh, max(ps, 1), 0 if kv_cache is None else 1)
         return q
 
-    DECODE_SPLIT = 256  # keys per decode work item (kSplit in attention_mfma.hip)
     PREFILL_TILE = 32  # tokens per prefill work item
+    DECODE_ITEMS = 1024  # decode attention: work items (wavefronts) to aim for
 
-    def attention_plan(self, seg_lens, seg_starts, retention, device):
+    def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1):
         """Work lists of the MFMA attention kernels for one step and one retention rule: the rows that are
-        single decode tokens, and tiles of up to 32 consecutive tokens of longer segments."""
+        single decode tokens (and into how many keys their work is split), and tiles of up to 32
+        consecutive tokens of longer segments."""
         from ..parts.base import first_needed_position
 
-        dec, tiles, max_splits = [], [], 1
+        dec, tiles, spans = [], [], []
         o = 0
         for n, start in zip(seg_lens, seg_starts):
             if n == 1:
                 dec.append(o)
-                first = first_needed_position(retention, start)
-                max_splits = max(max_splits, start // self.DECODE_SPLIT - first // self.DECODE_SPLIT + 1)
+                spans.append((first_needed_position(retention, start), start))
             else:
                 for t in range(0, n, self.PREFILL_TILE):
                     tiles += [o + t, min(self.PREFILL_TILE, n - t)]
             o += n
+        split, max_splits = 256, 1
+        if dec:
+            keys = sum(p - f + 1 for f, p in spans)
+            while split > 64 and keys * num_kv_heads // split < self.DECODE_ITEMS:
+                split //= 2
+            max_splits = max(p // split - f // split + 1 for f, p in spans)
         flat = torch.tensor(dec + tiles, dtype=torch.int32).to(device) if dec or tiles else None
-        return {"num_dec": len(dec), "num_tiles": len(tiles) // 2, "max_splits": max_splits,
+        return {"num_dec": len(dec), "num_tiles": len(tiles) // 2, "max_splits": max_splits, "split": split,
                 "dec": flat[: len(dec)] if dec else None, "tiles": flat[len(dec):] if tiles else None}
 
     def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
@@ -329,7 +336,7 @@ class HipOps:
                             seg_lens.append(0)
                             seg_starts.append(pos[i])
                         seg_lens[-1] += 1
-                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device)
+                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk)
                 if meta is not None:
                     meta.meta["attn_plan"] = plan
             if plan["num_tiles"]:
@@ -343,7 +350,7 @@ class HipOps:
                 ws_o = torch.empty(items * cols * dh, dtype=torch.float32, device=q.device)
                 self._call("jle_attention_decode", _p(q), _p(kv_cache), _p(out), _p(ws_ml), _p(ws_o), _p(positions),
                            _p(token_segment), _p(block_table), block_table.shape[1], _p(plan["dec"]), plan["num_dec"],
-                           plan["max_splits"], mode, param, float(scale), hq, hk, dh, ps)
+                           plan["max_splits"], plan["split"], mode, param, float(scale), hq, hk, dh, ps)
             return out
         self._call("jle_paged_attention_generic", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
                    _p(block_table), block_table.shape[1], mode, param, float(scale), self._is_bf16(q), n, hq, hk, dh,
