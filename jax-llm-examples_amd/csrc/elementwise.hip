@@ -165,19 +165,25 @@ JLE_API int jle_add_residual(float* x, const void* delta, int delta_is_bf16, lon
   return 0;
 }
 
-// ------------------------------------------------------------------ row gather (any dtype, rows of 4-byte words)
-__global__ void gather_rows_kernel(const uint32_t* __restrict__ src, const int* __restrict__ idx,
-                                   uint32_t* __restrict__ out, int words) {
-  const uint32_t* s = src + (size_t)idx[blockIdx.x] * words;
-  uint32_t* d = out + (size_t)blockIdx.x * words;
+// ------------------------------------------------------------------ row gather (any dtype)
+template <typename W>
+__global__ void gather_rows_kernel(const W* __restrict__ src, const int* __restrict__ idx, W* __restrict__ out,
+                                   int words) {
+  const W* s = src + (size_t)idx[blockIdx.x] * words;
+  W* d = out + (size_t)blockIdx.x * words;
   for (int i = threadIdx.x; i < words; i += blockDim.x) d[i] = s[i];
 }
 
 JLE_API int jle_gather_rows(const void* src, const int* idx, void* out, int M, int row_bytes, hipStream_t s) {
   if (M <= 0) return 0;
-  if (row_bytes % 4) return JLE_BAD_ARG;
-  hipLaunchKernelGGL(gather_rows_kernel, dim3(M), dim3(256), 0, s, (const uint32_t*)src, idx, (uint32_t*)out,
-                     row_bytes / 4);
+  if (row_bytes % 4 == 0)
+    hipLaunchKernelGGL(gather_rows_kernel<uint32_t>, dim3(M), dim3(256), 0, s, (const uint32_t*)src, idx,
+                       (uint32_t*)out, row_bytes / 4);
+  else if (row_bytes % 2 == 0)
+    hipLaunchKernelGGL(gather_rows_kernel<uint16_t>, dim3(M), dim3(256), 0, s, (const uint16_t*)src, idx,
+                       (uint16_t*)out, row_bytes / 2);
+  else
+    return JLE_BAD_ARG;
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -17,7 +17,7 @@ from jax_llm_examples_amd.engine.replay import make_runner
 from plain_llama4 import PlainModel
 from tiny_configs import TINY
 
-LENGTHS = {"A": [1, 80, 33, 47, 64, 9], "B": [120, 2, 49, 96, 31, 77], "C": [61, 40, 5, 83]}
+LENGTHS = {"A": [1, 80, 33, 47, 64, 9], "B": [120, 2, 49, 96, 31, 77], "C": [61, 40, 5, 83], "D": [37, 70, 3, 55, 64, 21]}
 MODES = {"whole": traces.whole, "tail": traces.tail, "portions": traces.portions, "mixed": traces.mixed}
 TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}  # of the largest logit of the request
 

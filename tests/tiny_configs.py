@@ -39,6 +39,20 @@ TINY = {
         "use_qk_norm": True, "attn_temperature_tuning": True, "floor_scale": 7, "attn_scale": 0.25,
         "rms_norm_eps": 1e-4, "tie_word_embeddings": False,
     },
+    # sizes that fit no fast path: a width that is no multiple of 4 or 8, expert width with 4 left over, a
+    # vocabulary that is prime, every head its own kv head, a chunk shorter than a page, NoPE first, dense first
+    "D": {
+        "architectures": ["Llama4ForCausalLM"],
+        "seed": 41,
+        "num_hidden_layers": 2, "hidden_size": 54, "num_attention_heads": 3, "num_key_value_heads": 3,
+        "head_dim": 16, "interleave_moe_layer_step": 2, "num_local_experts": 2, "num_experts_per_tok": 1,
+        "intermediate_size": 20, "intermediate_size_mlp": 28, "vocab_size": 257, "rope_theta": 50.0,
+        "rope_scaling": {"rope_type": "llama3", "factor": 2.0, "low_freq_factor": 1.0, "high_freq_factor": 2.0,
+                         "original_max_position_embeddings": 16},
+        "no_rope_layers": [0, 1], "attention_chunk_size": 7, "use_qk_norm": False,
+        "attn_temperature_tuning": True, "floor_scale": 5, "attn_scale": 0.3, "rms_norm_eps": 1e-3,
+        "tie_word_embeddings": False,
+    },
 }
 
 
