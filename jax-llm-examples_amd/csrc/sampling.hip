@@ -1,4 +1,4 @@
-// Next-token choice from float32 logits, one block per row.
+// Next-token choice from float32 logits.
 //   temperature == 0: the largest logit (lowest index among equals).
 //   temperature  > 0: Gumbel-max over logits / temperature, restricted to the top_k largest
 //                     (0 = all).  The noise of a token depends only on (seed, counter, token id),
@@ -49,47 +49,39 @@ __device__ __forceinline__ Best block_best(Best b, Best* smem) {
   return r;
 }
 
-__global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ logits,
-                                                     const float* __restrict__ temperature,
-                                                     const int* __restrict__ top_k, const int* __restrict__ seeds,
-                                                     const int* __restrict__ counters, int* __restrict__ out, int V) {
+__device__ __forceinline__ bool row_needs_threshold(float temp, int k, int V) { return temp > 0.f && k > 0 && k < V; }
+
+// Rows that sample among their top_k: one block per row.  First the threshold (the k-th largest of
+// x / temp, equal values counted separately, found by k passes), then Gumbel-max over what reaches it.
+__global__ __launch_bounds__(256) void sample_top_k_kernel(const float* __restrict__ logits,
+                                                           const float* __restrict__ temperature,
+                                                           const int* __restrict__ top_k,
+                                                           const int* __restrict__ seeds,
+                                                           const int* __restrict__ counters, int* __restrict__ out,
+                                                           int V) {
   __shared__ Best smem[4];
   const int row = blockIdx.x;
   const float* x = logits + (size_t)row * V;
   const float temp = temperature[row];
-  if (temp <= 0.f) {
+  const int k = top_k[row];
+  if (!row_needs_threshold(temp, k, V)) return;  // done by the two-stage kernels
+  float last_v = INFINITY;
+  int last_i = -1;
+  for (int it = 0; it < k; ++it) {
     Best b = {-INFINITY, 0x7fffffff};
-    for (int i = threadIdx.x; i < V; i += blockDim.x)
-      if (better(x[i], i, b.v, b.i)) {
-        b.v = x[i];
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+      const float z = x[i] / temp;
+      const bool after = z < last_v || (z == last_v && i > last_i);
+      if (after && better(z, i, b.v, b.i)) {
+        b.v = z;
         b.i = i;
       }
-    b = block_best(b, smem);
-    if (threadIdx.x == 0) out[row] = b.i == 0x7fffffff ? 0 : b.i;
-    return;
-  }
-  // threshold: the k-th largest of x / temp, counting equal values separately
-  float thr = -INFINITY;
-  const int k = top_k[row];
-  if (k > 0 && k < V) {
-    float last_v = INFINITY;
-    int last_i = -1;
-    for (int it = 0; it < k; ++it) {
-      Best b = {-INFINITY, 0x7fffffff};
-      for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        const float z = x[i] / temp;
-        const bool after = z < last_v || (z == last_v && i > last_i);
-        if (after && better(z, i, b.v, b.i)) {
-          b.v = z;
-          b.i = i;
-        }
-      }
-      b = block_best(b, smem);
-      last_v = b.v;
-      last_i = b.i;
     }
-    thr = last_v;
+    b = block_best(b, smem);
+    last_v = b.v;
+    last_i = b.i;
   }
+  const float thr = last_v;
   const uint32_t s = mix32((uint32_t)seeds[row] * 0x9E3779B1u + 0x85EBCA6Bu);
   const uint32_t c = mix32((((uint32_t)counters[row] + 1u) * 0xC2B2AE35u) ^ s);
   Best b = {-INFINITY, 0x7fffffff};
@@ -108,11 +100,93 @@ __global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ l
   if (threadIdx.x == 0) out[row] = b.i == 0x7fffffff ? 0 : b.i;
 }
 
+// Two stages for the rows that need one pass only (greedy, or temperature without top_k): each block
+// takes kChunk logits of one row, then one block per row picks among the blocks' choices.  The order
+// (value descending, index ascending) is total, so the result is that of a single pass.
+constexpr int kChunk = 8192;
+
+__global__ __launch_bounds__(256) void sample_partial_kernel(const float* __restrict__ logits,
+                                                             const float* __restrict__ temperature,
+                                                             const int* __restrict__ top_k,
+                                                             const int* __restrict__ seeds,
+                                                             const int* __restrict__ counters,
+                                                             float* __restrict__ part_v, int* __restrict__ part_i,
+                                                             int V, int S) {
+  __shared__ Best smem[4];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const float temp = temperature[row];
+  if (row_needs_threshold(temp, top_k[row], V)) return;
+  const float* x = logits + (size_t)row * V;
+  const int lo = chunk * kChunk, hi = min(V, lo + kChunk);
+  Best b = {-INFINITY, 0x7fffffff};
+  if (temp <= 0.f) {
+    for (int i = lo + threadIdx.x; i < hi; i += 256)
+      if (better(x[i], i, b.v, b.i)) {
+        b.v = x[i];
+        b.i = i;
+      }
+  } else {
+    const uint32_t s = mix32((uint32_t)seeds[row] * 0x9E3779B1u + 0x85EBCA6Bu);
+    const uint32_t c = mix32((((uint32_t)counters[row] + 1u) * 0xC2B2AE35u) ^ s);
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+      const float val = x[i] / temp + (-logf(-logf(uniform_from_hash(s, c, (uint32_t)i))));
+      if (better(val, i, b.v, b.i)) {
+        b.v = val;
+        b.i = i;
+      }
+    }
+  }
+  b = block_best(b, smem);
+  if (threadIdx.x == 0) {
+    part_v[(size_t)row * S + chunk] = b.v;
+    part_i[(size_t)row * S + chunk] = b.i;
+  }
+}
+
+__global__ __launch_bounds__(64) void sample_final_kernel(const float* __restrict__ temperature,
+                                                          const int* __restrict__ top_k,
+                                                          const float* __restrict__ part_v,
+                                                          const int* __restrict__ part_i, int* __restrict__ out, int V,
+                                                          int S) {
+  const int row = blockIdx.x;
+  if (row_needs_threshold(temperature[row], top_k[row], V)) return;
+  Best b = {-INFINITY, 0x7fffffff};
+  for (int s = threadIdx.x; s < S; s += 64) {
+    const float v = part_v[(size_t)row * S + s];
+    const int i = part_i[(size_t)row * S + s];
+    if (better(v, i, b.v, b.i)) {
+      b.v = v;
+      b.i = i;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(b.v, o, 64);
+    const int oi = __shfl_xor(b.i, o, 64);
+    if (better(ov, oi, b.v, b.i)) {
+      b.v = ov;
+      b.i = oi;
+    }
+  }
+  if (threadIdx.x == 0) out[row] = b.i == 0x7fffffff ? 0 : b.i;
+}
+
+// part_v / part_i: workspaces of M * ceil(V / 8192) entries.  any_top_k: 0 if the caller knows that no row
+// samples among its top_k (then the one-block-per-row kernel is not launched at all).
 JLE_API int jle_sample(const float* logits, const float* temperature, const int* top_k, const int* seeds,
-                       const int* counters, int* out, int M, int V, hipStream_t s) {
+                       const int* counters, int* out, float* part_v, int* part_i, int M, int V, int any_top_k,
+                       hipStream_t s) {
   if (M <= 0) return 0;
-  if (V <= 0) return JLE_BAD_ARG;
-  hipLaunchKernelGGL(sample_kernel, dim3(M), dim3(256), 0, s, logits, temperature, top_k, seeds, counters, out, V);
+  if (V <= 0 || M > 65535) return JLE_BAD_ARG;
+  const int S = (V + kChunk - 1) / kChunk;
+  hipLaunchKernelGGL(sample_partial_kernel, dim3(S, M), dim3(256), 0, s, logits, temperature, top_k, seeds, counters,
+                     part_v, part_i, V, S);
   JLE_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sample_final_kernel, dim3(M), dim3(64), 0, s, temperature, top_k, part_v, part_i, out, V, S);
+  JLE_LAUNCH_CHECK();
+  if (any_top_k) {
+    hipLaunchKernelGGL(sample_top_k_kernel, dim3(M), dim3(256), 0, s, logits, temperature, top_k, seeds, counters, out, V);
+    JLE_LAUNCH_CHECK();
+  }
   return 0;
 }

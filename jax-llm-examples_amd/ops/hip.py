@@ -29,7 +29,7 @@ _SIGNATURES = {
     "jle_moe_route": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-    "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
     "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
     "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i,
@@ -404,12 +404,16 @@ class HipOps:
         return ExpertSum(routed, inv, k, shared, n, d)
 
     # ------------------------------------------------------------------ sampling
-    def sample(self, logits, temperature, top_k, seeds, counters):
+    def sample(self, logits, temperature, top_k, seeds, counters, any_top_k: bool = True):
         m, v = logits.shape
         self._chk(logits, torch.float32, None, "logits")
         self._chk(temperature, torch.float32, (m,), "temperature")
         for t, what in ((top_k, "top_k"), (seeds, "seeds"), (counters, "counters")):
             self._chk(t, torch.int32, (m,), what)
         out = torch.empty(m, dtype=torch.int32, device=logits.device)
-        self._call("jle_sample", _p(logits), _p(temperature), _p(top_k), _p(seeds), _p(counters), _p(out), m, v)
+        chunks = -(-v // 8192)
+        part_v = torch.empty(m * chunks, dtype=torch.float32, device=logits.device)
+        part_i = torch.empty(m * chunks, dtype=torch.int32, device=logits.device)
+        self._call("jle_sample", _p(logits), _p(temperature), _p(top_k), _p(seeds), _p(counters), _p(out), _p(part_v),
+                   _p(part_i), m, v, int(any_top_k))
         return out

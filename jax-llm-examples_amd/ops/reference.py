@@ -184,7 +184,7 @@ class ReferenceOps:
         return out
 
     # ------------------------------------------------------------------ sampling
-    def sample(self, logits, temperature, top_k, seeds, counters):
+    def sample(self, logits, temperature, top_k, seeds, counters, any_top_k: bool = True):
         """Greedy where ``temperature == 0`` (lowest index among equals); otherwise
         Gumbel-max over ``logits / temperature`` restricted to the ``top_k`` largest
         (0 = all), with noise that depends only on (seed, counter, token id)."""

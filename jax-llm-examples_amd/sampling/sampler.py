@@ -23,5 +23,7 @@ class Sampler:
         seeds = torch.tensor([int(p.seed) & 0x7FFFFFFF for p in params], dtype=torch.int32)
         ctr = torch.tensor([int(c) & 0x7FFFFFFF for c in counters], dtype=torch.int32)
         dev = self.device
-        out = self.ops.sample(logits, temp.to(dev), topk.to(dev), seeds.to(dev), ctr.to(dev))
+        packed = torch.stack([topk, seeds, ctr]).to(dev)  # one copy for the three integer rows
+        any_top_k = any(not p.greedy and 0 < p.sample_topk for p in params)
+        out = self.ops.sample(logits, temp.to(dev), packed[0], packed[1], packed[2], any_top_k=any_top_k)
         return [int(t) for t in out.cpu().tolist()]
