@@ -273,6 +273,8 @@ class HipOps:
             ps = kv_cache.shape[3]
             self._chk(kv_cache, qkv.dtype, (kv_cache.shape[0], 2, hk, ps, dh), "kv pages")
             self._chk(slot_mapping, torch.int32, (n,), "slot mapping")
+        if dh % 2 or dh > 512:
+            raise KernelError(f"rotary/norm kernel: head size {dh} must be even and at most 512")
         q = torch.empty(n, hq, dh, dtype=qkv.dtype, device=qkv.device)
         fs, sc = (query_scale if query_scale is not None else (0.0, 0.0))
         self._call("jle_qk_prepare", _p(qkv), _p(q), _p(kv_cache), _p(positions),
@@ -352,6 +354,10 @@ class HipOps:
                            _p(token_segment), _p(block_table), block_table.shape[1], _p(plan["dec"]), plan["num_dec"],
                            plan["max_splits"], plan["split"], mode, param, float(scale), hq, hk, dh, ps)
             return out
+        if dh % 8 or dh > 256:
+            raise KernelError(f"attention kernels: head size {dh} is not supported (a multiple of 8, at most 256)")
+        if hq % hk:
+            raise KernelError(f"attention kernels: {hq} query heads are no multiple of {hk} kv heads")
         self._call("jle_paged_attention_generic", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
                    _p(block_table), block_table.shape[1], mode, param, float(scale), self._is_bf16(q), n, hq, hk, dh,
                    ps)
@@ -363,6 +369,8 @@ class HipOps:
         e = router.shape[0]
         self._chk(h32, torch.float32, None, "router input")
         self._chk(router, torch.float32, (e, d), "router matrix")
+        if not 1 <= top_k <= min(8, e) or e > 4096:
+            raise KernelError(f"router kernel: top_k {top_k} of {e} experts is not supported (top_k <= 8, experts <= 4096)")
         ids = torch.empty(n, top_k, dtype=torch.int32, device=h32.device)
         gates = torch.empty(n, top_k, dtype=torch.float32, device=h32.device)
         logits = torch.empty(n, e, dtype=torch.float32, device=h32.device)

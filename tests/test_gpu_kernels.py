@@ -160,8 +160,10 @@ def test_paged_attention(ops, ref, dt, hq, hk, dh, ps, retention):
 def test_attention_refuses_a_head_size_it_cannot_do(ops):
     from jax_llm_examples_amd.ops.hip import KernelError
     q, kv, bt, pos, seg = _attention_case(2, 1, 20, 16, torch.float32, [(0, 4)])
-    with pytest.raises(KernelError, match="refuses"):
+    with pytest.raises(KernelError, match="head size 20 is not supported"):
         ops.paged_attention(q, kv, bt, pos, seg, ("all",), 1.0)
+    with pytest.raises(KernelError, match="top_k 9"):
+        ops.moe_route(torch.zeros(2, 64, device=DEV), torch.zeros(16, 64, device=DEV), 9)
 
 
 @pytest.mark.parametrize("dt", DT)
