@@ -22,6 +22,7 @@ constexpr int BM = 128;    // rows of X per block
 constexpr int BN = 128;    // rows of W per block
 constexpr int BK = 64;     // K per step (32 was measured slower: more barriers per product)
 constexpr int PITCH = 72;  // elements between rows in shared memory (64 + 8): 16-byte reads of 16 rows hit all banks
+constexpr int NS = 2;      // register sets of tiles on their way from memory (3 measured the same, 4 slower: one block per CU)
 constexpr int CPT = BM * BK / 8 / 256;  // 16-byte chunks per thread and matrix
 constexpr int CPR = BK / 8;             // chunks per row
 
@@ -111,9 +112,9 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
     const int src = xok[i] ? (a_rows != nullptr ? a_rows[tok] : tok) : 0;
     xsrc[i] = X + (size_t)src * K + kc;
   }
-  // two register sets: the tile two steps ahead is on its way while the tile one step ahead waits to be
-  // written to shared memory, so a load has two steps of matrix work to arrive
-  uint4 wreg[2][CPT], xreg[2][CPT];
+  // NS register sets: at step kt the tile kt + NS is asked for, so a load has NS - 1 steps of matrix work
+  // to arrive before it is written to shared memory
+  uint4 wreg[NS][CPT], xreg[NS][CPT];
   auto load_tile = [&](int set, int k0) {
     const bool kok = k0 + kc < K;  // K is a multiple of 8
 #pragma unroll
@@ -144,9 +145,10 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
   const int nk = (K + BK - 1) / BK;
   load_tile(0, 0);
   store_tile(0, 0);
-  if (nk > 1) load_tile(1, BK);
+#pragma unroll
+  for (int s = 1; s < NS; ++s)
+    if (s < nk) load_tile(s, s * BK);
   __syncthreads();
-  // the loop is unrolled by two so that the register sets are named at compile time
   auto compute = [&](int buf) {
     if (!wave_has_rows) return;
 #pragma unroll
@@ -168,18 +170,19 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
         for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[i], acc[j][i], 0, 0, 0);
     }
   };
-  for (int kt = 0; kt < nk; kt += 2) {
-    // even step: tile kt is in buffer 0, tile kt + 1 in register set 1
-    if (kt + 2 < nk) load_tile(0, (kt + 2) * BK);
-    compute(0);
-    if (kt + 1 < nk) store_tile(1, 1);
-    __syncthreads();
-    if (kt + 1 >= nk) break;
-    // odd step: tile kt + 1 is in buffer 1, tile kt + 2 in register set 0
-    if (kt + 3 < nk) load_tile(1, (kt + 3) * BK);
-    compute(1);
-    if (kt + 2 < nk) store_tile(0, 0);
-    __syncthreads();
+  // unrolled by NS so that the register sets are named at compile time; at step kt: tile kt is in shared
+  // buffer kt & 1, tiles kt + 1 .. kt + NS - 1 are in (or on their way to) sets (kt + 1) % NS ..
+  for (int kt0 = 0; kt0 < nk; kt0 += NS) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int kt = kt0 + s;
+      if (kt < nk) {
+        if (kt + NS < nk) load_tile(s, (kt + NS) * BK);  // set s held tile kt, which is in shared memory now
+        compute(kt & 1);
+        if (kt + 1 < nk) store_tile((s + 1) % NS, (kt + 1) & 1);
+        __syncthreads();
+      }
+    }
   }
   if (!wave_has_rows) return;
 

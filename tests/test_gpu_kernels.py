@@ -194,6 +194,34 @@ def test_attention_finds_one_far_key_among_hundreds_and_respects_the_window_edge
     assert run(599, ("window", W)).abs().max() < 1.0
 
 
+@pytest.mark.parametrize("dt", DT)
+def test_attention_portion_sees_a_far_key_exactly_where_the_rule_allows(ops, dt):
+    """The same with a portion of 40 tokens (positions 660..699) in one step: with a chunk of 96 the tokens
+    before 672 are in the chunk that starts at 576, the others in the one that starts at 672; with a window
+    of 100 each token has its own edge."""
+    hq, hk, dh, ps = 4, 2, 32, 16
+    q, kv, bt, pos, seg = _attention_case(hq, hk, dh, ps, dt, [(660, 40)], seed=4)
+    q.zero_()
+    q[:, :, 0] = 8.0
+
+    def run(hot, retention):
+        k = kv.clone()
+        k[:, 0] *= 0.05
+        page, off = int(bt[0, hot // ps]), hot % ps
+        k[page, 0, :, off, 0] = 8.0
+        k[page, 1].view(hk, dh, ps)[:, :, off] = 3.0
+        return ops.paged_attention(q, k, bt, pos, seg, retention, 1.0).float().abs().amin(dim=-1)  # per token
+
+    def sees(out):
+        return [bool(v > 2.9) for v in out.tolist()]
+
+    assert sees(run(5, ("all",))) == [True] * 40
+    assert sees(run(576, ("chunk", 96))) == [p < 672 for p in range(660, 700)]
+    assert sees(run(575, ("chunk", 96))) == [False] * 40
+    assert sees(run(672, ("chunk", 96))) == [p >= 672 for p in range(660, 700)]  # causal: not before its own position
+    assert sees(run(580, ("window", 100))) == [p - 99 <= 580 for p in range(660, 700)]
+
+
 def test_attention_reading_a_page_that_was_given_back_is_not_silent(ops):
     q, kv, bt, pos, seg = _attention_case(2, 1, 16, 16, torch.float32, [(40, 1)])
     bt[0, 1] = -1
