@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
                                                            OutT* __restrict__ Y, const int* __restrict__ offsets,
                                                            const int* __restrict__ a_rows,
                                                            const float* __restrict__ scale, int M, int Nout, int K,
-                                                           int G) {
+                                                           int G, int tiled) {
   __shared__ __attribute__((aligned(16))) bf16_t sW[2][BN * PITCH];
   __shared__ __attribute__((aligned(16))) bf16_t sX[2][BM * PITCH];
   // which group and which of its rows
@@ -106,7 +106,10 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
     } else {
       wrow = min(n0 + rr, Nout - 1);
     }
-    wsrc[i] = We + (size_t)wrow * K + kc;
+    if (tiled)  // tile (wrow / 16, k / 32) of 512 elements; inside it element ((k % 32) / 8 * 16 + wrow % 16) * 8
+      wsrc[i] = We + ((size_t)(wrow >> 4) * (K >> 5) + (kc >> 5)) * 512 + (((kc & 31) >> 3) * 16 + (wrow & 15)) * 8;
+    else
+      wsrc[i] = We + (size_t)wrow * K + kc;
     const int tok = row0 + rr;
     xok[i] = tok < row_end;
     const int src = xok[i] ? (a_rows != nullptr ? a_rows[tok] : tok) : 0;
@@ -115,13 +118,14 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
   // NS register sets: at step kt the tile kt + NS is asked for, so a load has NS - 1 steps of matrix work
   // to arrive before it is written to shared memory
   uint4 wreg[NS][CPT], xreg[NS][CPT];
+  const int wstep = tiled ? 16 : 1;  // a step of 64 k is two tiles of 512 elements in the streaming layout
   auto load_tile = [&](int set, int k0) {
     const bool kok = k0 + kc < K;  // K is a multiple of 8
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
       wreg[set][i] = uint4{0u, 0u, 0u, 0u};
       xreg[set][i] = uint4{0u, 0u, 0u, 0u};
-      if (kok) wreg[set][i] = *reinterpret_cast<const uint4*>(wsrc[i] + k0);
+      if (kok) wreg[set][i] = *reinterpret_cast<const uint4*>(wsrc[i] + (size_t)k0 * wstep);
       if (kok && xok[i]) xreg[set][i] = *reinterpret_cast<const uint4*>(xsrc[i] + k0);
     }
   };
@@ -232,16 +236,17 @@ __global__ __launch_bounds__(256) void gemm_grouped_kernel(const bf16_t* __restr
 // X [*, K] bf16, W [G, Nout, K] bf16, Y [M, Nout] (or [M, Nout / 2] with swiglu) bf16 or float32
 JLE_API int jle_gemm_grouped(const void* X, const void* W, void* Y, const int* offsets, const int* a_rows,
                              const float* scale, int swiglu, int out_f32, int M, int Nout, int K, int G,
-                             hipStream_t s) {
+                             int tiled, hipStream_t s) {
   if (M <= 0 || Nout <= 0) return 0;
   if (K <= 0 || K % 8 || G < 1 || (swiglu && Nout % 2)) return JLE_BAD_ARG;
+  if (tiled && (K % 32 || Nout % 16)) return JLE_BAD_ARG;
   const int row_tiles = (M + BM - 1) / BM + (offsets != nullptr ? G : 0);
   if (row_tiles > 65535) return JLE_BAD_ARG;
   const int xtiles = swiglu ? (Nout / 2 + BN / 2 - 1) / (BN / 2) : (Nout + BN - 1) / BN;
   dim3 g(xtiles, row_tiles), b(256);
 #define LAUNCH(SW, OT)                                                                                     \
   hipLaunchKernelGGL((gemm_grouped_kernel<SW, OT>), g, b, 0, s, (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, \
-                     offsets, a_rows, scale, M, Nout, K, G)
+                     offsets, a_rows, scale, M, Nout, K, G, tiled)
   if (swiglu) {
     if (out_f32) LAUNCH(true, float); else LAUNCH(true, bf16_t);
   } else {

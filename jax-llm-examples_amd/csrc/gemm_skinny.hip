@@ -11,6 +11,10 @@
 // shared memory in a fixed order.  Each block owns two 16-row weight tiles (SWIGLU: the gate tile
 // and its up tile, so the activation is formed in the epilogue); grid = (row tiles, token tiles,
 // groups); blocks of groups without rows leave at once.
+//
+// W is either row-major or in the streaming layout (`tiled`): tiles of 16 rows x 32 k stored as the
+// kilobyte one A-operand load reads (lane g * 16 + r: row r, elements 8 g ..), tiles along K
+// contiguous - then every load instruction of a wavefront reads one contiguous kilobyte.
 #include "common.h"
 
 using namespace jle;
@@ -38,7 +42,8 @@ template <int MT, bool SWIGLU, typename OutT, int WAVES, int kUnroll, int RT = 2
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W,
                                                           OutT* __restrict__ Y, const int* __restrict__ offsets,
                                                           const int* __restrict__ a_rows,
-                                                          const float* __restrict__ scale, int M, int Nout, int K) {
+                                                          const float* __restrict__ scale, int M, int Nout, int K,
+                                                          int tiled) {
   static_assert(RT == 2 || !SWIGLU, "the fused activation needs the gate tile and the up tile");
   __shared__ float red[WAVES][RT * MT * 4][64];
   const int e = blockIdx.z;
@@ -62,8 +67,22 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     ra0 = min(base + r, Nout - 1);
     ra1 = min(base + 16 + r, Nout - 1);
   }
-  const bf16_t* a0 = We + (size_t)ra0 * K + g * 8;
-  const bf16_t* a1 = We + (size_t)ra1 * K + g * 8;
+  const int nkb = (K + 31) >> 5;
+  const bf16_t* a0;
+  const bf16_t* a1;
+  int kb_stride;  // elements from one k-block of 32 to the next
+  if (tiled) {  // rows and K are whole tiles
+    const int ntile = Nout >> 4;
+    const int t0 = SWIGLU ? (base >> 4) : min(base >> 4, ntile - 1);
+    const int t1 = SWIGLU ? ((half + base) >> 4) : min((base >> 4) + 1, ntile - 1);
+    a0 = We + (size_t)t0 * nkb * 512 + lane * 8;
+    a1 = We + (size_t)t1 * nkb * 512 + lane * 8;
+    kb_stride = 512;
+  } else {
+    a0 = We + (size_t)ra0 * K + g * 8;
+    a1 = We + (size_t)ra1 * K + g * 8;
+    kb_stride = 32;
+  }
   const bf16_t* xb[MT];
   bool xv[MT];
 #pragma unroll
@@ -79,15 +98,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     acc0[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     acc1[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  const int nkb = (K + 31) >> 5;
   for (int kb0 = wave; kb0 < nkb; kb0 += WAVES * kUnroll) {
     bf16x8 A0[kUnroll], A1[kUnroll], B[kUnroll][MT];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int kb = kb0 + WAVES * u;
       const bool ok = kb < nkb && (kb * 32 + g * 8) < K;  // K is a multiple of 8
-      A0[u] = ok ? load8(a0 + kb * 32) : zero8();
-      if (RT == 2) A1[u] = ok ? load8(a1 + kb * 32) : zero8();
+      A0[u] = ok ? load8(a0 + (size_t)kb * kb_stride) : zero8();
+      if (RT == 2) A1[u] = ok ? load8(a1 + (size_t)kb * kb_stride) : zero8();
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) B[u][mt] = (ok && xv[mt]) ? load8(xb[mt] + kb * 32) : zero8();
     }
@@ -149,12 +167,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 // variant = row tiles * 256 + wavefronts * 16 + unroll
 template <int MT, bool SW, typename OT>
 static int launch_skinny(int xrows, int ytiles, int G, hipStream_t s, int variant, const void* X, const void* W,
-                         void* Y, const int* offsets, const int* a_rows, const float* scale, int M, int Nout, int K) {
+                         void* Y, const int* offsets, const int* a_rows, const float* scale, int M, int Nout, int K,
+                         int tiled) {
 #define LAUNCH(RT, WV, UN)                                                                                       \
   do {                                                                                                           \
     dim3 g((xrows + 16 * (SW ? 1 : RT) - 1) / (16 * (SW ? 1 : RT)), ytiles, G);                                  \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, SW, OT, WV, UN, (SW ? 2 : RT)>), g, dim3(WV * 64), 0, s,          \
-                       (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, offsets, a_rows, scale, M, Nout, K);          \
+                       (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, offsets, a_rows, scale, M, Nout, K, tiled);   \
     return 0;                                                                                                    \
   } while (0)
   switch (variant) {
@@ -175,9 +194,10 @@ static int launch_skinny(int xrows, int ytiles, int G, hipStream_t s, int varian
 // max_rows: the most rows any group can have (M if unknown).  variant: 0 = chosen from the sizes.
 JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* offsets, const int* a_rows,
                             const float* scale, int swiglu, int out_f32, int M, int Nout, int K, int G, int max_rows,
-                            int variant, hipStream_t s) {
+                            int variant, int tiled, hipStream_t s) {
   if (M <= 0 || Nout <= 0) return 0;
   if (K <= 0 || K % 8 || G < 1 || G > 65535 || (swiglu && Nout % 2)) return JLE_BAD_ARG;
+  if (tiled && (K % 32 || Nout % 16 || (swiglu && (Nout / 2) % 16))) return JLE_BAD_ARG;
   if (max_rows <= 0 || max_rows > M) max_rows = M;
   const int mt = (offsets == nullptr && max_rows > 32) ? 4 : (offsets == nullptr && max_rows > 16) ? 2 : 1;
   const int ytiles = (max_rows + 16 * mt - 1) / (16 * mt);
@@ -194,9 +214,9 @@ JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* of
   int rc;
 #define PICK(SW, OT)                                                                                             \
   do {                                                                                                           \
-    if (mt == 1) rc = launch_skinny<1, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K);      \
-    else if (mt == 2) rc = launch_skinny<2, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K); \
-    else rc = launch_skinny<4, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K);              \
+    if (mt == 1) rc = launch_skinny<1, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled);      \
+    else if (mt == 2) rc = launch_skinny<2, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled); \
+    else rc = launch_skinny<4, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled);              \
   } while (0)
   if (swiglu) {
     if (out_f32) PICK(true, float); else PICK(true, bf16_t);

@@ -34,8 +34,8 @@ _SIGNATURES = {
     "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
     "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i,
                              _vp],
-    "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
 
@@ -206,7 +206,7 @@ class HipOps:
     SKINNY_DENSE_ROWS = 16  # the fused gate|up projection of a dense feed-forward: beyond this the BLAS library
 
     def gemm_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
-                    variant=0):
+                    variant=0, tiled=False):
         """bfloat16 weight-streaming product on MFMA for few rows (see ``gemm_skinny.hip``); with ``swiglu`` the
         result is ``silu(gate) * up`` of the two halves of ``b``'s rows."""
         if b.dim() == 2:
@@ -222,10 +222,11 @@ class HipOps:
         out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
                           device=a.device)
         self._call("jle_gemm_skinny", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
-                   int(out_f32), m, nout, k, g, m, variant)
+                   int(out_f32), m, nout, k, g, m, variant, int(tiled))
         return out
 
-    def gemm_grouped(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None):
+    def gemm_grouped(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
+                     tiled=False):
         """bfloat16 product on MFMA for many rows, grouped by ``offsets`` (see ``gemm_grouped.hip``)."""
         if b.dim() == 2:
             b = b.unsqueeze(0)
@@ -240,16 +241,17 @@ class HipOps:
         out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
                           device=a.device)
         self._call("jle_gemm_grouped", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
-                   int(out_f32), m, nout, k, g)
+                   int(out_f32), m, nout, k, g, int(tiled))
         return out
 
-    def lm_head(self, h, w):
+    def lm_head(self, h, w, tiled: bool = False):
+        """float32 logits; ``tiled``: ``w`` is in the streaming layout (``ops/layout.py``)."""
         if h.dtype == torch.float32:
             return torch.matmul(h, w.t())
         if h.shape[1] % 8 == 0:
             if h.shape[0] <= self.SKINNY_MAX_ROWS:
-                return self.gemm_skinny(h, w, out_f32=True)
-            return self.gemm_grouped(h, w, out_f32=True)
+                return self.gemm_skinny(h, w, out_f32=True, tiled=tiled)
+            return self.gemm_grouped(h, w, out_f32=True, tiled=tiled)
         return self.gemm(h, w, out_f32=True)
 
     def silu_mul(self, gate_up):
@@ -391,18 +393,22 @@ class HipOps:
                    m, num_experts, k)
         return offsets, sorted_token, sorted_gate, inv
 
-    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None):
+    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False):
         n, d = h.shape
         e, f2, _ = w_gate_up.shape
         k = expert_ids.shape[1]
         offsets, sorted_token, sorted_gate, inv = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e)
         mfma = h.dtype == torch.bfloat16 and d % 8 == 0 and (f2 // 2) % 8 == 0
         if mfma and n * k <= 2 * self.SKINNY_MAX_ROWS:  # few rows: the cost is streaming the chosen experts' weights
-            act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True)
-            routed = self.gemm_skinny(act, w_down, offsets=offsets)
+            act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,
+                                   tiled=tiled)
+            routed = self.gemm_skinny(act, w_down, offsets=offsets, tiled=tiled)
         elif mfma:
-            act = self.gemm_grouped(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True)
-            routed = self.gemm_grouped(act, w_down, offsets=offsets)
+            act = self.gemm_grouped(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,
+                                    tiled=tiled)
+            routed = self.gemm_grouped(act, w_down, offsets=offsets, tiled=tiled)
+        elif tiled:
+            raise KernelError("weights in the streaming layout need the MFMA product kernels")
         else:
             gu = self.gemm(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate)
             act = self.silu_mul(gu)

@@ -63,7 +63,8 @@ class ReferenceOps:
         out = h.float() @ w.float().t()
         return out.to(out_dtype or h.dtype)
 
-    def lm_head(self, h, w):
+    def lm_head(self, h, w, tiled: bool = False):
+        assert not tiled, "the plain ops read row-major weights"
         return h.float() @ w.float().t()
 
     def swiglu_linear(self, h, w_gate_up):
@@ -164,11 +165,12 @@ class ReferenceOps:
         vals = torch.gather(logits, 1, order)
         return order.to(torch.int32), torch.sigmoid(vals)
 
-    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None):
+    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False):
         """``sum_j  W_down[e_j] (silu(g_j W_gate[e_j] h) * (g_j W_up[e_j] h))`` per token,
         plus ``shared`` if given; float32 result.  ``w_gate_up`` is ``[E, 2F, D]`` (gate rows then
         up rows), ``w_down`` ``[E, D, F]``.  Activations between the two products are
         rounded to the run dtype, as the kernels store them."""
+        assert not tiled, "the plain ops read row-major weights"
         n, d = h.shape
         f = w_down.shape[2]
         out = torch.zeros(n, d, dtype=torch.float32, device=h.device)

@@ -46,6 +46,7 @@ class MoESigmoidShared(FeedForward):
         self.inter = int(spec.intermediate_size)
         self.shared_inter = int(spec.get("shared_intermediate_size") or 0)
         self.last_routing = None  # (expert ids, gates) of the latest call, for tests
+        self.tiled = False  # expert matrices are in the kernels' streaming layout (ops/layout.py)
 
     def param_specs(self):
         e, f, d = self.num_experts, self.inter, self.hidden
@@ -59,6 +60,15 @@ class MoESigmoidShared(FeedForward):
             specs["shared_down"] = ParamSpec((d, self.shared_inter))
         return specs
 
+    def finalize(self) -> None:
+        from ..ops.layout import can_tile, tile_
+
+        gu, dn = self.params["w_gate_up"], self.params["w_down"]
+        if not self.tiled and can_tile(gu) and can_tile(dn) and self.inter % 16 == 0:
+            tile_(gu)
+            tile_(dn)
+            self.tiled = True
+
     def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
         ops = ctx.ops
         expert_ids, gates = ops.moe_route(h32, self.params["router"], self.top_k)
@@ -70,4 +80,5 @@ class MoESigmoidShared(FeedForward):
         shared = None
         if self.shared_inter:
             shared = ops.linear(ops.swiglu_linear(h, self.params["shared_gate_up"]), self.params["shared_down"])
-        return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"], shared)
+        return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"], shared,
+                               tiled=self.tiled)

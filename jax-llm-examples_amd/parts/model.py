@@ -21,6 +21,19 @@ class _Table(Part):
         return {"weight": ParamSpec(self.shape)}
 
 
+class _Head(_Table):
+    """The output head: its matrix takes the product kernels' streaming layout where it can."""
+
+    tiled = False
+
+    def finalize(self) -> None:
+        from ..ops.layout import can_tile, tile_
+
+        if not self.tiled and can_tile(self.params["weight"]):
+            tile_(self.params["weight"])
+            self.tiled = True
+
+
 class DecoderModel:
     def __init__(self, plan: ModelPlan, dtype: torch.dtype, device) -> None:
         self.plan = plan
@@ -29,7 +42,7 @@ class DecoderModel:
         self.embed = _Table(plan.vocab_size, plan.hidden_size)
         self.blocks = [build_block(spec) for spec in plan.layers]
         self.final_norm = build_norm(plan.final_norm)
-        self.lm_head = None if plan.tie_word_embeddings else _Table(plan.vocab_size, plan.hidden_size)
+        self.lm_head = None if plan.tie_word_embeddings else _Head(plan.vocab_size, plan.hidden_size)
         self._allocated = False
 
     # ------------------------------------------------------------------ parameters
@@ -101,4 +114,4 @@ class DecoderModel:
         picked = residual.rows(ctx, ctx.logits_indices)
         h, _ = self.final_norm.forward(picked, ctx)
         head = self.embed if self.lm_head is None else self.lm_head
-        return ops.lm_head(h, head.params["weight"])
+        return ops.lm_head(h, head.params["weight"], tiled=getattr(head, "tiled", False))

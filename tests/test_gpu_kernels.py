@@ -417,3 +417,35 @@ def test_grouped_product_for_many_rows(ops, ref, n, d, f, e, k):
     assert float((dense - h.float() @ wgu[0].float().t()).abs().max() / dense.abs().max()) <= 2e-5
     head = ops.lm_head(h[:100, :], _rand(311, d, dt=dt, seed=7))
     assert head.dtype == torch.float32 and head.shape == (100, 311)
+
+
+def test_streaming_layout_gives_the_same_results_bit_for_bit(ops):
+    from jax_llm_examples_amd.ops.layout import can_tile, tile_, untiled
+    dt = torch.bfloat16
+    w = _rand(3, 96, 160, dt=dt, seed=1)
+    wt = w.clone()
+    assert can_tile(w) and not can_tile(_rand(3, 90, 160, dt=dt)) and not can_tile(w.float())
+    tile_(wt)
+    assert not torch.equal(wt, w) and torch.equal(untiled(wt), w)
+    first_tile = wt[1].flatten()[:512].reshape(4, 16, 8)  # the first kilobyte: rows 0..15, k 0..31 as [g][r][8]
+    assert torch.equal(first_tile[2, 5], w[1, 5, 16:24])
+    second = wt[1].flatten()[512:1024].reshape(4, 16, 8)  # the next tile goes on along K
+    assert torch.equal(second[0, 3], w[1, 3, 32:40])
+    for n, d, f, e, k in [(8, 128, 48, 16, 1), (50, 160, 96, 5, 2), (400, 256, 64, 4, 1)]:
+        h = _rand(n, d, dt=dt, seed=1)
+        wgu, wd = _rand(e, 2 * f, d, dt=dt, scale=0.1, seed=2), _rand(e, d, f * 1, dt=dt, scale=0.1, seed=3)
+        if f % 32:
+            continue
+        g = torch.Generator().manual_seed(5)
+        ids = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(n)]).to(torch.int32).to(DEV)
+        gates = torch.rand(n, k, generator=g).to(DEV)
+        wgu_t, wd_t = wgu.clone(), wd.clone()
+        tile_(wgu_t), tile_(wd_t)
+        a = ops.materialize(ops.moe_experts(h, ids, gates, wgu, wd, None))
+        b = ops.materialize(ops.moe_experts(h, ids, gates, wgu_t, wd_t, None, tiled=True))
+        assert torch.equal(a, b)
+    for m in (3, 40, 200):
+        h, w2 = _rand(m, 160, dt=dt, seed=4), _rand(17 * 16, 160, dt=dt, seed=5)  # an odd number of row tiles
+        w2t = w2.clone()
+        tile_(w2t)
+        assert torch.equal(ops.lm_head(h, w2), ops.lm_head(h, w2t, tiled=True))
