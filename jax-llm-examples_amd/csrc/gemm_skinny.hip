@@ -209,7 +209,7 @@ JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* of
     const long long pair_tiles = (long long)((xrows + (swiglu ? 15 : 31)) / (swiglu ? 16 : 32)) * groups;
     if (swiglu) variant = 2 * 256 + 4 * 16 + 8;
     else if (pair_tiles >= 4096) variant = 2 * 256 + 4 * 16 + 8;  // very many rows of W (the output head)
-    else variant = 1 * 256 + 8 * 16 + 4;  // one row tile per block, 8 wavefronts split K: more blocks in flight
+    else variant = 1 * 256 + 4 * 16 + 8;  // one row tile per block: more blocks in flight
   }
   int rc;
 #define PICK(SW, OT)                                                                                             \
