@@ -50,6 +50,85 @@ struct Columns {  // per lane, for each of its column tiles
   int lo, hi;     // keys this column may read within the wave's range (inclusive); lo > hi: none
 };
 
+// One step of 32 keys for the columns of a wavefront: mask the scores, update the running maximum and sum,
+// turn the scores into the B operand of the second product and add V^T P^T to the accumulators.
+//   st[ct][tt]: scores of key tile tt (keys kb + 16 tt + 4 g + i in element i); act0 / act1: the tile exists
+//   vraw[dt]: for element row 16 dt + (lane % 16): keys 4 g .. 4 g + 3 of tile 0 (x, y) and of tile 1 (z, w)
+template <int DH, int CT>
+__device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], bool act0, bool act1,
+                                                   const uint4 (&vraw)[DH / 16], int kb, const Columns (&col)[CT],
+                                                   int k_lo, int k_hi, float scale_log2, float (&m)[CT],
+                                                   float (&l)[CT], f32x4 (&acc)[CT][DH / 16]) {
+  constexpr int DT = DH / 16;
+  const int g = (threadIdx.x & 63) >> 4;
+  // mask, running max and sum per column
+  bf16x8 pb[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    float s[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + 16 * tt + 4 * g + i;
+        const bool ok = (tt == 0 ? act0 : act1) && key >= col[ct].lo && key <= col[ct].hi;
+        const float v = ok ? st[ct][tt][i] * scale_log2 : -INFINITY;
+        s[tt * 4 + i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m[ct], mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = exp2f(m[ct] - m_use);  // m = -inf: 0 (nothing accumulated yet)
+    float sum = 0.f;
+    float p[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      p[j] = exp2f(s[j] - m_use);  // masked: exp2(-inf) = 0
+      sum += p[j];
+    }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    l[ct] = l[ct] * corr + sum;
+    m[ct] = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      acc[ct][dt][0] *= corr;
+      acc[ct][dt][1] *= corr;
+      acc[ct][dt][2] *= corr;
+      acc[ct][dt][3] *= corr;
+    }
+    const uint4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+    pb[ct] = __builtin_bit_cast(bf16x8, pk);
+  }
+  // values: keys outside [k_lo, k_hi] may never have been written: they are read as zero
+  uint32_t keep[2][2];  // per tile, per pair of keys: which halves to keep
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int key = kb + 16 * tt + 4 * g + 2 * h2;
+      const uint32_t lo_ok = (key >= k_lo && key <= k_hi) ? 0x0000ffffu : 0u;
+      const uint32_t hi_ok = (key + 1 >= k_lo && key + 1 <= k_hi) ? 0xffff0000u : 0u;
+      keep[tt][h2] = lo_ok | hi_ok;
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    uint4 vv = vraw[dt];
+    vv.x &= keep[0][0];
+    vv.y &= keep[0][1];
+    vv.z &= keep[1][0];
+    vv.w &= keep[1][1];
+    const bf16x8 a = __builtin_bit_cast(bf16x8, vv);
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+      acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct], acc[ct][dt], 0, 0, 0);
+  }
+}
+
 // The shared core.  DH: head size; CT: column tiles.  Returns through m, l, acc (O^T, unnormalised).
 template <int DH, int CT>
 __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv,
@@ -148,72 +227,7 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
     }
     // the next step's keys (overwrites kraw, vbase and active: this step keeps act0 / act1 and vraw)
     if (kb + 32 <= k_hi) locate_and_load_keys(kb + 32);
-    // mask, running max and sum per column
-    bf16x8 pb[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-      float s[8];
-      float mx = -INFINITY;
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = kb + 16 * tt + 4 * g + i;
-          const bool ok = (tt == 0 ? act0 : act1) && key >= col[ct].lo && key <= col[ct].hi;
-          const float v = ok ? st[ct][tt][i] * scale_log2 : -INFINITY;
-          s[tt * 4 + i] = v;
-          mx = fmaxf(mx, v);
-        }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[ct], mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float corr = exp2f(m[ct] - m_use);  // m = -inf: 0 (nothing accumulated yet)
-      float sum = 0.f;
-      float p[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        p[j] = exp2f(s[j] - m_use);  // masked: exp2(-inf) = 0
-        sum += p[j];
-      }
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
-      l[ct] = l[ct] * corr + sum;
-      m[ct] = m_new;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        acc[ct][dt][0] *= corr;
-        acc[ct][dt][1] *= corr;
-        acc[ct][dt][2] *= corr;
-        acc[ct][dt][3] *= corr;
-      }
-      const uint4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
-      pb[ct] = __builtin_bit_cast(bf16x8, pk);
-    }
-    // values: keys outside [k_lo, k_hi] may never have been written: they are read as zero
-    uint32_t keep[2][2];  // per tile, per pair of keys: which halves to keep
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-#pragma unroll
-      for (int h2 = 0; h2 < 2; ++h2) {
-        const int key = kb + 16 * tt + 4 * g + 2 * h2;
-        const uint32_t lo_ok = (key >= k_lo && key <= k_hi) ? 0x0000ffffu : 0u;
-        const uint32_t hi_ok = (key + 1 >= k_lo && key + 1 <= k_hi) ? 0xffff0000u : 0u;
-        keep[tt][h2] = lo_ok | hi_ok;
-      }
-    }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      uint4 vv = vraw[dt];
-      vv.x &= keep[0][0];
-      vv.y &= keep[0][1];
-      vv.z &= keep[1][0];
-      vv.w &= keep[1][1];
-      const bf16x8 a = __builtin_bit_cast(bf16x8, vv);
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
-        acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct], acc[ct][dt], 0, 0, 0);
-    }
+    softmax_and_values<DH, CT>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
   }
 }
 
@@ -261,6 +275,175 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     bf16_t* o = out + ((size_t)col[ct].token * Hq + h) * DH + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < DH / 16; ++dt) {
+      const uint2 v = {pack_bf16(acc[ct][dt][0] * inv, acc[ct][dt][1] * inv),
+                       pack_bf16(acc[ct][dt][2] * inv, acc[ct][dt][3] * inv)};
+      *reinterpret_cast<uint2*>(o + dt * 16) = v;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ prefill portions, heads sharing keys
+// One block per (tile of up to 32 tokens, kv head, up to WAVES of its query heads): a wavefront per
+// query head.  The heads read the same keys and values, so every 32-key step is brought into shared
+// memory once by the whole block (the next step's data is in flight meanwhile) and each wavefront
+// takes its operands from there.  Keys get a row pitch of DH + 8 elements (16-byte reads of 16 rows then
+// hit all banks); values keep the page's layout [DH][16].
+template <int DH, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
+    const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
+    int table_width, const int* __restrict__ tiles, int num_tiles, int ret_mode, int ret_param, float scale_log2,
+    int Hq, int Hkv, int ps) {
+  constexpr int CT = 2, KC = DH / 32, DT = DH / 16;
+  constexpr int KP = DH + 8;
+  constexpr int THREADS = WAVES * 64;
+  constexpr int NCH = 8 * DH;                             // 16-byte chunks per step: K 2 x 16 x DH / 8, V the same
+  constexpr int CPT = (NCH + THREADS - 1) / THREADS;      // per thread
+  __shared__ __attribute__((aligned(16))) bf16_t sK[2][32 * KP];
+  __shared__ __attribute__((aligned(16))) bf16_t sV[2][2 * DH * 16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c16 = lane & 15, g = lane >> 4;
+  const int G = Hq / Hkv;
+  const int hchunks = (G + WAVES - 1) / WAVES;
+  const int hc = blockIdx.x % hchunks;
+  const int hk = (blockIdx.x / hchunks) % Hkv;
+  const int tile = num_tiles - 1 - blockIdx.x / (hchunks * Hkv);  // the tiles with the most keys first
+  const int gi = hc * WAVES + wave;
+  const bool head_ok = gi < G;
+  const int h = hk * G + (head_ok ? gi : 0);
+  const int n0 = tiles[2 * tile], nt = tiles[2 * tile + 1];
+  const int p_first = positions[n0], p_last = p_first + nt - 1;
+  const int k_lo = first_key(ret_mode, ret_param, p_first);
+  const int k_hi = p_last;
+  const int* table = block_table + (size_t)token_segment[n0] * table_width;
+  const size_t plane = (size_t)ps * DH;
+  const size_t page_stride = 2 * (size_t)Hkv * plane;
+
+  Columns col[CT];
+  bf16x8 qb[CT][KC];
+  float m[CT], l[CT];
+  f32x4 acc[CT][DT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = ct * 16 + c16;
+    const bool ok = c < nt && head_ok;
+    const int pos = p_first + c;
+    col[ct].token = c < nt ? n0 + c : n0;
+    col[ct].head = h;
+    col[ct].lo = ok ? first_key(ret_mode, ret_param, pos) : 1;
+    col[ct].hi = ok ? pos : 0;
+    const bf16_t* qrow = q + ((size_t)col[ct].token * Hq + h) * DH + g * 8;
+#pragma unroll
+    for (int c2 = 0; c2 < KC; ++c2) {
+      uint4 v = {0u, 0u, 0u, 0u};
+      if (ok) v = *reinterpret_cast<const uint4*>(qrow + c2 * 32);
+      qb[ct][c2] = __builtin_bit_cast(bf16x8, v);
+    }
+    m[ct] = -INFINITY;
+    l[ct] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  bool bad = false;
+  uint4 reg[CPT];
+  bool act_next[2] = {false, false};
+  // asks for the chunks of step kb (into reg) and notes which of its two key tiles exist
+  auto load_step = [&](int kb) {
+    const bf16_t* kplane[2];  // the page's key plane of this kv head; its value plane is Hkv planes further
+    int off[2];               // the tile's first key within the page
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const int key0 = kb + 16 * tt;
+      bool a = key0 <= k_hi && key0 + 15 >= k_lo;
+      int page = -1;
+      if (a) {
+        page = table[key0 / ps];
+        if (page < 0) {
+          bad = true;
+          a = false;
+        }
+      }
+      act_next[tt] = a;
+      kplane[tt] = a ? kv + (size_t)page * page_stride + (size_t)hk * plane : nullptr;
+      off[tt] = key0 % ps;
+    }
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int c = threadIdx.x + THREADS * i;
+      reg[i] = uint4{0u, 0u, 0u, 0u};
+      if (c < NCH) {
+        const int which = c / (2 * DH), idx = c % (2 * DH);  // 0, 1: key tiles; 2, 3: value tiles
+        const int tt = which & 1;
+        if (kplane[tt] != nullptr) {
+          const bf16_t* src;
+          if (which < 2)  // keys: row idx / (DH / 8) of the tile, 8 elements from (idx % (DH / 8)) * 8
+            src = kplane[tt] + (size_t)(off[tt] + idx / (DH / 8)) * DH + (idx % (DH / 8)) * 8;
+          else  // values: element row idx / 2, keys (idx % 2) * 8 .. + 7 of the tile
+            src = kplane[tt] + (size_t)Hkv * plane + (size_t)(idx >> 1) * ps + off[tt] + (idx & 1) * 8;
+          reg[i] = *reinterpret_cast<const uint4*>(src);
+        }
+      }
+    }
+  };
+  auto store_step = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int c = threadIdx.x + THREADS * i;
+      if (c < NCH) {
+        const int which = c / (2 * DH), idx = c % (2 * DH);
+        const int tt = which & 1;
+        if (which < 2)
+          *reinterpret_cast<uint4*>(&sK[buf][(tt * 16 + idx / (DH / 8)) * KP + (idx % (DH / 8)) * 8]) = reg[i];
+        else
+          *reinterpret_cast<uint4*>(&sV[buf][(tt * DH + (idx >> 1)) * 16 + (idx & 1) * 8]) = reg[i];
+      }
+    }
+  };
+
+  const int kb_first = (k_lo / 32) * 32;
+  int buf = 0;
+  if (kb_first <= k_hi) load_step(kb_first);
+  for (int kb = kb_first; kb <= k_hi; kb += 32) {
+    const bool act0 = act_next[0], act1 = act_next[1];
+    store_step(buf);
+    __syncthreads();
+    if (kb + 32 <= k_hi) load_step(kb + 32);
+    if (head_ok) {
+      f32x4 st[CT][2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+          const uint4 kvv = *reinterpret_cast<const uint4*>(&sK[buf][(tt * 16 + c16) * KP + c * 32 + g * 8]);
+          const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct)
+            st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
+        }
+      }
+      uint4 vraw[DT];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const uint2 t0 = *reinterpret_cast<const uint2*>(&sV[buf][(0 * DH + dt * 16 + c16) * 16 + 4 * g]);
+        const uint2 t1 = *reinterpret_cast<const uint2*>(&sV[buf][(1 * DH + dt * 16 + c16) * 16 + 4 * g]);
+        vraw[dt] = uint4{t0.x, t0.y, t1.x, t1.y};
+      }
+      softmax_and_values<DH, CT>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+    }
+    buf ^= 1;
+  }
+  if (!head_ok) return;
+  bad = __any(bad);
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    if (ct * 16 + c16 >= nt) continue;
+    const float inv = bad ? __builtin_nanf("") : (l[ct] > 0.f ? 1.0f / l[ct] : 0.f);
+    bf16_t* o = out + ((size_t)col[ct].token * Hq + h) * DH + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
       const uint2 v = {pack_bf16(acc[ct][dt][0] * inv, acc[ct][dt][1] * inv),
                        pack_bf16(acc[ct][dt][2] * inv, acc[ct][dt][3] * inv)};
       *reinterpret_cast<uint2*>(o + dt * 16) = v;
@@ -363,18 +546,54 @@ JLE_API int jle_attention_mfma_supported(int dh, int Hq, int Hkv, int ps) {
 
 JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, const int* positions,
                                   const int* token_segment, const int* block_table, int table_width, const int* tiles,
-                                  int num_tiles, int ret_mode, int ret_param, float scale, int Hq, int Hkv, int dh,
-                                  int ps, hipStream_t s) {
+                                  int num_tiles, int tile_tokens, int ret_mode, int ret_param, float scale, int Hq,
+                                  int Hkv, int dh, int ps, hipStream_t s) {
   if (num_tiles <= 0) return 0;
   if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps)) return JLE_BAD_ARG;
   if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
   const long long items = (long long)num_tiles * Hq;
   dim3 g((unsigned)((items + 3) / 4)), b(256);
   const float sl = scale * kLog2e;
-#define LAUNCH(DH)                                                                                                 \
-  hipLaunchKernelGGL((attention_prefill_kernel<DH, 2>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,           \
-                     (bf16_t*)out, positions, token_segment, block_table, table_width, tiles, num_tiles, ret_mode, \
-                     ret_param, sl, Hq, Hkv, ps)
+  if (tile_tokens != 16 && tile_tokens != 32) return JLE_BAD_ARG;
+  const int G = Hq / Hkv;
+  if (G >= 2 && tile_tokens == 32) {
+    const int waves = G <= 2 ? 2 : G <= 4 ? 4 : G == 5 ? 5 : 8;
+    const int hchunks = (G + waves - 1) / waves;
+    dim3 gs((unsigned)((long long)num_tiles * Hkv * hchunks));
+#define LAUNCH_S(DH, WV)                                                                                          \
+  hipLaunchKernelGGL((attention_prefill_shared_kernel<DH, WV>), gs, dim3(WV * 64), 0, s, (const bf16_t*)q,        \
+                     (const bf16_t*)kv, (bf16_t*)out, positions, token_segment, block_table, table_width, tiles,  \
+                     num_tiles, ret_mode, ret_param, sl, Hq, Hkv, ps)
+#define PICK_S(DH)                    \
+  do {                                \
+    if (waves == 2) LAUNCH_S(DH, 2);  \
+    else if (waves == 4) LAUNCH_S(DH, 4); \
+    else if (waves == 5) LAUNCH_S(DH, 5); \
+    else LAUNCH_S(DH, 8);             \
+  } while (0)
+    switch (dh) {
+      case 32: PICK_S(32); break;
+      case 64: PICK_S(64); break;
+      case 96: PICK_S(96); break;
+      case 128: PICK_S(128); break;
+      case 256: PICK_S(256); break;
+    }
+#undef PICK_S
+#undef LAUNCH_S
+    JLE_LAUNCH_CHECK();
+    return 0;
+  }
+#define LAUNCH(DH)                                                                                                   \
+  do {                                                                                                               \
+    if (tile_tokens == 32)                                                                                           \
+      hipLaunchKernelGGL((attention_prefill_kernel<DH, 2>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,         \
+                         (bf16_t*)out, positions, token_segment, block_table, table_width, tiles, num_tiles,         \
+                         ret_mode, ret_param, sl, Hq, Hkv, ps);                                                      \
+    else                                                                                                             \
+      hipLaunchKernelGGL((attention_prefill_kernel<DH, 1>), g, b, 0, s, (const bf16_t*)q, (const bf16_t*)kv,         \
+                         (bf16_t*)out, positions, token_segment, block_table, table_width, tiles, num_tiles,         \
+                         ret_mode, ret_param, sl, Hq, Hkv, ps);                                                      \
+  } while (0)
   switch (dh) {
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;

@@ -31,7 +31,7 @@ _SIGNATURES = {
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
-    "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
+    "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
     "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i,
                              _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -285,7 +285,7 @@ class HipOps:
                    n, hq, hk, dh, max(ps, 1), 0 if kv_cache is None else 1)
         return q
 
-    PREFILL_TILE = 32  # tokens per prefill work item
+    PREFILL_TILE = int(__import__("os").environ.get("JLE_PREFILL_TILE", "32"))  # tokens per prefill work item
     DECODE_ITEMS = 1024  # decode attention: work items (wavefronts) to aim for
 
     def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1):
@@ -345,8 +345,8 @@ class HipOps:
                     meta.meta["attn_plan"] = plan
             if plan["num_tiles"]:
                 self._call("jle_attention_prefill", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
-                           _p(block_table), block_table.shape[1], _p(plan["tiles"]), plan["num_tiles"], mode, param,
-                           float(scale), hq, hk, dh, ps)
+                           _p(block_table), block_table.shape[1], _p(plan["tiles"]), plan["num_tiles"],
+                           self.PREFILL_TILE, mode, param, float(scale), hq, hk, dh, ps)
             if plan["num_dec"]:
                 cols = 16 if hq // hk <= 16 else 32
                 items = plan["num_dec"] * hk * plan["max_splits"]
