@@ -25,6 +25,8 @@
 // range is one work item and leaves (max, sum, unnormalised O); a second kernel merges them in
 // order.  Which ranges and tiles a query visits depends only on its position, the retention rule
 // and `split`.
+#include <limits.h>
+
 #include "common.h"
 
 using namespace jle;
@@ -40,29 +42,49 @@ __device__ __forceinline__ int first_key(int mode, int param, int pos) {
   return 0;
 }
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
-}
-
 struct Columns {  // per lane, for each of its column tiles
   int token;      // row of q / out
   int head;       // query head
   int lo, hi;     // keys this column may read within the wave's range (inclusive); lo > hi: none
 };
 
-// One step of 32 keys for the columns of a wavefront: mask the scores, update the running maximum and sum,
-// turn the scores into the B operand of the second product and add V^T P^T to the accumulators.
+// Maximum / sum over the four lanes that hold one column (equal lane % 16), in all of them.  The two swaps
+// exchange the halves of the wavefront and neighbouring rows of 16 lanes: no trip through shared memory.
+__device__ __forceinline__ float column_max(float v) {
+  uint32_t u = __float_as_uint(v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  u = __float_as_uint(v);
+  r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+__device__ __forceinline__ float column_sum(float v) {
+  uint32_t u = __float_as_uint(v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  u = __float_as_uint(v);
+  r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// One step of 32 keys for the columns of a wavefront: mask the scores (MASKED; without it every key of the
+// step is known to be visible to every live column), update the running maximum and sum, turn the scores
+// into the B operand of the second product and add V^T P^T to the accumulators.  Both forms do the same
+// arithmetic on a visible key.
 //   st[ct][tt]: scores of key tile tt (keys kb + 16 tt + 4 g + i in element i); act0 / act1: the tile exists
 //   vraw[dt]: for element row 16 dt + (lane % 16): keys 4 g .. 4 g + 3 of tile 0 (x, y) and of tile 1 (z, w)
-template <int DH, int CT>
+//   l: each lane's own part of the column's sum (column_sum at the end gives the whole)
+template <int DH, int CT, bool MASKED>
 __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], bool act0, bool act1,
                                                    const uint4 (&vraw)[DH / 16], int kb, const Columns (&col)[CT],
                                                    int k_lo, int k_hi, float scale_log2, float (&m)[CT],
                                                    float (&l)[CT], f32x4 (&acc)[CT][DH / 16]) {
   constexpr int DT = DH / 16;
   const int g = (threadIdx.x & 63) >> 4;
-  // mask, running max and sum per column
   bf16x8 pb[CT];
+  float corr[CT];
+  bool unchanged = true;
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     float s[8];
@@ -71,61 +93,96 @@ __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], boo
     for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = kb + 16 * tt + 4 * g + i;
-        const bool ok = (tt == 0 ? act0 : act1) && key >= col[ct].lo && key <= col[ct].hi;
-        const float v = ok ? st[ct][tt][i] * scale_log2 : -INFINITY;
+        float v = st[ct][tt][i];
+        if (MASKED) {
+          const int key = kb + 16 * tt + 4 * g + i;
+          const bool ok = (tt == 0 ? act0 : act1) && key >= col[ct].lo && key <= col[ct].hi;
+          v = ok ? v : -INFINITY;
+        }
         s[tt * 4 + i] = v;
         mx = fmaxf(mx, v);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m[ct], mx);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = exp2f(m[ct] - m_use);  // m = -inf: 0 (nothing accumulated yet)
+    mx = column_max(mx);
+    const float m_new = fmaxf(m[ct], mx * scale_log2);  // the scale is positive
+    const float m_use = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
+    corr[ct] = __builtin_amdgcn_exp2f(m[ct] - m_use);  // m = -inf: 0 (nothing accumulated yet)
+    unchanged = unchanged && m_new == m[ct];
     float sum = 0.f;
     float p[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      p[j] = exp2f(s[j] - m_use);  // masked: exp2(-inf) = 0
+      p[j] = __builtin_amdgcn_exp2f(fmaf(s[j], scale_log2, -m_use));  // masked: exp2(-inf) = 0
       sum += p[j];
     }
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
-    l[ct] = l[ct] * corr + sum;
+    l[ct] = l[ct] * corr[ct] + sum;
     m[ct] = m_new;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      acc[ct][dt][0] *= corr;
-      acc[ct][dt][1] *= corr;
-      acc[ct][dt][2] *= corr;
-      acc[ct][dt][3] *= corr;
-    }
     const uint4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
     pb[ct] = __builtin_bit_cast(bf16x8, pk);
   }
-  // values: keys outside [k_lo, k_hi] may never have been written: they are read as zero
-  uint32_t keep[2][2];  // per tile, per pair of keys: which halves to keep
-#pragma unroll
-  for (int tt = 0; tt < 2; ++tt) {
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-      const int key = kb + 16 * tt + 4 * g + 2 * h2;
-      const uint32_t lo_ok = (key >= k_lo && key <= k_hi) ? 0x0000ffffu : 0u;
-      const uint32_t hi_ok = (key + 1 >= k_lo && key + 1 <= k_hi) ? 0xffff0000u : 0u;
-      keep[tt][h2] = lo_ok | hi_ok;
-    }
-  }
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt) {
-    uint4 vv = vraw[dt];
-    vv.x &= keep[0][0];
-    vv.y &= keep[0][1];
-    vv.z &= keep[1][0];
-    vv.w &= keep[1][1];
-    const bf16x8 a = __builtin_bit_cast(bf16x8, vv);
+  // no column of the wavefront has a new maximum: every factor is exactly one (or the sums are still zero)
+  if (!__all(unchanged)) {
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
-      acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct], acc[ct][dt], 0, 0, 0);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        acc[ct][dt][0] *= corr[ct];
+        acc[ct][dt][1] *= corr[ct];
+        acc[ct][dt][2] *= corr[ct];
+        acc[ct][dt][3] *= corr[ct];
+      }
+  }
+  if (MASKED) {
+    // values: keys outside [k_lo, k_hi] may never have been written: they are read as zero
+    uint32_t keep[2][2];  // per tile, per pair of keys: which halves to keep
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const int key = kb + 16 * tt + 4 * g + 2 * h2;
+        const uint32_t lo_ok = (key >= k_lo && key <= k_hi) ? 0x0000ffffu : 0u;
+        const uint32_t hi_ok = (key + 1 >= k_lo && key + 1 <= k_hi) ? 0xffff0000u : 0u;
+        keep[tt][h2] = lo_ok | hi_ok;
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint4 vv = vraw[dt];
+      vv.x &= keep[0][0];
+      vv.y &= keep[0][1];
+      vv.z &= keep[1][0];
+      vv.w &= keep[1][1];
+      const bf16x8 a = __builtin_bit_cast(bf16x8, vv);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct], acc[ct][dt], 0, 0, 0);
+    }
+  } else {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const bf16x8 a = __builtin_bit_cast(bf16x8, vraw[dt]);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct], acc[ct][dt], 0, 0, 0);
+    }
+  }
+}
+
+// The widest range of keys that every live column of the wavefront may read: a step of 32 keys inside
+// [lo, hi] needs no mask.  Columns without keys (lo > hi: padding, whose results nobody stores) do not count.
+template <int CT>
+__device__ __forceinline__ void common_range(const Columns (&col)[CT], int& lo, int& hi) {
+  lo = INT_MIN;
+  hi = INT_MAX;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct)
+    if (col[ct].lo <= col[ct].hi) {
+      lo = max(lo, col[ct].lo);
+      hi = min(hi, col[ct].hi);
+    }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    lo = max(lo, __shfl_xor(lo, o, 64));
+    hi = min(hi, __shfl_xor(hi, o, 64));
   }
 }
 
@@ -190,6 +247,8 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
       }
     }
   };
+  int all_lo, all_hi;
+  common_range<CT>(col, all_lo, all_hi);
   const int kb_first = (k_lo / 32) * 32;
   if (kb_first <= k_hi) locate_and_load_keys(kb_first);
   for (int kb = kb_first; kb <= k_hi; kb += 32) {
@@ -227,8 +286,13 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
     }
     // the next step's keys (overwrites kraw, vbase and active: this step keeps act0 / act1 and vraw)
     if (kb + 32 <= k_hi) locate_and_load_keys(kb + 32);
-    softmax_and_values<DH, CT>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+    if (__all(act0 && act1 && kb >= all_lo && kb + 31 <= all_hi))
+      softmax_and_values<DH, CT, false>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+    else
+      softmax_and_values<DH, CT, true>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
   }
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) l[ct] = column_sum(l[ct]);
 }
 
 // ------------------------------------------------------------------ prefill portions
@@ -297,10 +361,10 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
   constexpr int CT = 2, KC = DH / 32, DT = DH / 16;
   constexpr int KP = DH + 8;
   constexpr int THREADS = WAVES * 64;
-  constexpr int NCH = 8 * DH;                             // 16-byte chunks per step: K 2 x 16 x DH / 8, V the same
-  constexpr int CPT = (NCH + THREADS - 1) / THREADS;      // per thread
-  __shared__ __attribute__((aligned(16))) bf16_t sK[2][32 * KP];
-  __shared__ __attribute__((aligned(16))) bf16_t sV[2][2 * DH * 16];
+  constexpr int NCH = 8 * DH;                         // 16-byte chunks per step: keys 2 x 16 x DH / 8, values the same
+  constexpr int CPT = (NCH + THREADS - 1) / THREADS;  // per thread
+  constexpr int SK = 32 * KP, SV = 2 * DH * 16;       // elements of a buffer: keys, then values
+  __shared__ __attribute__((aligned(16))) bf16_t smem[2][SK + SV];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c16 = lane & 15, g = lane >> 4;
   const int G = Hq / Hkv;
@@ -344,103 +408,146 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
+  int all_lo, all_hi;
+  common_range<CT>(col, all_lo, all_hi);
+
+  // Who brings what.  Chunk c of a step belongs to key tile c & 1 (THREADS is even, so all chunks of a
+  // thread are of one tile and the thread follows one page); within the tile, r = c >> 1 < 2 DH is a
+  // piece of the keys (row r / (DH / 8), 8 elements from (r % (DH / 8)) * 8), the rest a piece of the
+  // values (element row (r - 2 DH) / 2, keys ((r - 2 DH) % 2) * 8 .. + 7 of the tile).
+  const int my_tile = threadIdx.x & 1;
+  int src_off[CPT];  // elements from the tile's first key (keys) or first value column (values)
+  int dst_off[CPT];  // elements within a buffer
+  bool is_key[CPT], in_use[CPT];
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int c = threadIdx.x + THREADS * i;
+    const int r = c >> 1;
+    in_use[i] = c < NCH;
+    is_key[i] = r < 2 * DH;
+    if (is_key[i]) {
+      src_off[i] = (r / (DH / 8)) * DH + (r % (DH / 8)) * 8;
+      dst_off[i] = (my_tile * 16 + r / (DH / 8)) * KP + (r % (DH / 8)) * 8;
+    } else {
+      const int r2 = r - 2 * DH;
+      src_off[i] = (r2 >> 1) * ps + (r2 & 1) * 8;
+      dst_off[i] = SK + (my_tile * DH + (r2 >> 1)) * 16 + (r2 & 1) * 8;
+    }
+  }
 
   bool bad = false;
-  uint4 reg[CPT];
-  bool act_next[2] = {false, false};
-  // asks for the chunks of step kb (into reg) and notes which of its two key tiles exist
-  auto load_step = [&](int kb) {
-    const bf16_t* kplane[2];  // the page's key plane of this kv head; its value plane is Hkv planes further
-    int off[2];               // the tile's first key within the page
+  // PF register sets: the data of the next PF steps are on their way while a step is worked on
+  constexpr int PF = 2;
+  uint4 reg[PF][CPT];
+  // The cursor: the next step to ask for (the same in all threads, so the block table is read through the
+  // scalar path, which the wait for the bulk loads does not include).  The pages of a step are looked up
+  // when the step before it is asked for.
+  const int kb_first = (k_lo / 32) * 32;
+  int next_kb = kb_first;
+  int page_index = next_kb / ps, page_off = next_kb % ps;  // of the step's first key
+  int pages[2], offs[2];                                   // per key tile: page (-1: none) and first key within it
+  auto look_up = [&]() {
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      const int key0 = kb + 16 * tt;
-      bool a = key0 <= k_hi && key0 + 15 >= k_lo;
-      int page = -1;
-      if (a) {
-        page = table[key0 / ps];
-        if (page < 0) {
-          bad = true;
-          a = false;
-        }
+      const int key0 = next_kb + 16 * tt;
+      int idx = page_index, off = page_off + 16 * tt;
+      if (off >= ps) {
+        off -= ps;
+        ++idx;
       }
-      act_next[tt] = a;
-      kplane[tt] = a ? kv + (size_t)page * page_stride + (size_t)hk * plane : nullptr;
-      off[tt] = key0 % ps;
-    }
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int c = threadIdx.x + THREADS * i;
-      reg[i] = uint4{0u, 0u, 0u, 0u};
-      if (c < NCH) {
-        const int which = c / (2 * DH), idx = c % (2 * DH);  // 0, 1: key tiles; 2, 3: value tiles
-        const int tt = which & 1;
-        if (kplane[tt] != nullptr) {
-          const bf16_t* src;
-          if (which < 2)  // keys: row idx / (DH / 8) of the tile, 8 elements from (idx % (DH / 8)) * 8
-            src = kplane[tt] + (size_t)(off[tt] + idx / (DH / 8)) * DH + (idx % (DH / 8)) * 8;
-          else  // values: element row idx / 2, keys (idx % 2) * 8 .. + 7 of the tile
-            src = kplane[tt] + (size_t)Hkv * plane + (size_t)(idx >> 1) * ps + off[tt] + (idx & 1) * 8;
-          reg[i] = *reinterpret_cast<const uint4*>(src);
-        }
+      offs[tt] = off;
+      pages[tt] = -1;
+      if (key0 <= k_hi && key0 + 15 >= k_lo) {
+        pages[tt] = table[idx];
+        if (pages[tt] < 0) bad = true;  // the tile is then read as zeros, and the block's result is NaN
       }
     }
   };
-  auto store_step = [&](int buf) {
+  look_up();
+  auto load_step = [&](int set) {
+    const int page = my_tile ? pages[1] : pages[0];
+    const int off = my_tile ? offs[1] : offs[0];
+    const bf16_t* keys = kv + (size_t)(page < 0 ? 0 : page) * page_stride + (size_t)hk * plane;
+    const bf16_t* values = keys + (size_t)Hkv * plane + off;
+    keys += (size_t)off * DH;
 #pragma unroll
     for (int i = 0; i < CPT; ++i) {
-      const int c = threadIdx.x + THREADS * i;
-      if (c < NCH) {
-        const int which = c / (2 * DH), idx = c % (2 * DH);
-        const int tt = which & 1;
-        if (which < 2)
-          *reinterpret_cast<uint4*>(&sK[buf][(tt * 16 + idx / (DH / 8)) * KP + (idx % (DH / 8)) * 8]) = reg[i];
-        else
-          *reinterpret_cast<uint4*>(&sV[buf][(tt * DH + (idx >> 1)) * 16 + (idx & 1) * 8]) = reg[i];
-      }
+      reg[set][i] = uint4{0u, 0u, 0u, 0u};
+      if (in_use[i] && page >= 0)
+        reg[set][i] = *reinterpret_cast<const uint4*>((is_key[i] ? keys : values) + src_off[i]);
     }
+    next_kb += 32;
+    page_off += 32;  // a page holds at least 16 keys: at most two pages further
+    if (page_off >= ps) {
+      page_off -= ps;
+      ++page_index;
+    }
+    if (page_off >= ps) {
+      page_off -= ps;
+      ++page_index;
+    }
+    look_up();
+  };
+  auto store_step = [&](int set, int buf) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i)
+      if (in_use[i]) *reinterpret_cast<uint4*>(&smem[buf][dst_off[i]]) = reg[set][i];
   };
 
-  const int kb_first = (k_lo / 32) * 32;
   int buf = 0;
-  if (kb_first <= k_hi) load_step(kb_first);
-  for (int kb = kb_first; kb <= k_hi; kb += 32) {
-    const bool act0 = act_next[0], act1 = act_next[1];
-    store_step(buf);
-    __syncthreads();
-    if (kb + 32 <= k_hi) load_step(kb + 32);
-    if (head_ok) {
-      f32x4 st[CT][2];
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
+  for (int s2 = 0; s2 < PF; ++s2)
+    if (kb_first + 32 * s2 <= k_hi) load_step(s2);
+  // unrolled by PF so that the register sets are named at compile time: step kb0 + 32 s2 is in set s2
+  for (int kb0 = kb_first; kb0 <= k_hi; kb0 += 32 * PF) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s2 = 0; s2 < PF; ++s2) {
+      const int kb = kb0 + 32 * s2;
+      if (kb <= k_hi) {
+        store_step(s2, buf);
+        __syncthreads();
+        if (kb + 32 * PF <= k_hi) load_step(s2);
+        if (head_ok) {
+          const bf16_t* sK = smem[buf];
+          const bf16_t* sV = smem[buf] + SK;
+          f32x4 st[CT][2];
 #pragma unroll
-        for (int c = 0; c < KC; ++c) {
-          const uint4 kvv = *reinterpret_cast<const uint4*>(&sK[buf][(tt * 16 + c16) * KP + c * 32 + g * 8]);
-          const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
+          for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
-          for (int ct = 0; ct < CT; ++ct)
-            st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
+            for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+              const uint4 kvv = *reinterpret_cast<const uint4*>(&sK[(tt * 16 + c16) * KP + c * 32 + g * 8]);
+              const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
+#pragma unroll
+              for (int ct = 0; ct < CT; ++ct)
+                st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
+            }
+          }
+          uint4 vraw[DT];
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const uint2 t0 = *reinterpret_cast<const uint2*>(&sV[(0 * DH + dt * 16 + c16) * 16 + 4 * g]);
+            const uint2 t1 = *reinterpret_cast<const uint2*>(&sV[(1 * DH + dt * 16 + c16) * 16 + 4 * g]);
+            vraw[dt] = uint4{t0.x, t0.y, t1.x, t1.y};
+          }
+          if (kb >= all_lo && kb + 31 <= all_hi) {  // the same for the whole wavefront
+            softmax_and_values<DH, CT, false>(st, true, true, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+          } else {
+            const bool act0 = kb <= k_hi && kb + 15 >= k_lo, act1 = kb + 16 <= k_hi && kb + 31 >= k_lo;
+            softmax_and_values<DH, CT, true>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+          }
         }
+        buf ^= 1;
       }
-      uint4 vraw[DT];
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const uint2 t0 = *reinterpret_cast<const uint2*>(&sV[buf][(0 * DH + dt * 16 + c16) * 16 + 4 * g]);
-        const uint2 t1 = *reinterpret_cast<const uint2*>(&sV[buf][(1 * DH + dt * 16 + c16) * 16 + 4 * g]);
-        vraw[dt] = uint4{t0.x, t0.y, t1.x, t1.y};
-      }
-      softmax_and_values<DH, CT>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
     }
-    buf ^= 1;
   }
   if (!head_ok) return;
-  bad = __any(bad);
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     if (ct * 16 + c16 >= nt) continue;
-    const float inv = bad ? __builtin_nanf("") : (l[ct] > 0.f ? 1.0f / l[ct] : 0.f);
+    const float sum = column_sum(l[ct]);
+    const float inv = bad ? __builtin_nanf("") : (sum > 0.f ? 1.0f / sum : 0.f);
     bf16_t* o = out + ((size_t)col[ct].token * Hq + h) * DH + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -506,11 +613,15 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   }
 }
 
-// Merges a decode token's key ranges, in order.  One block of DH threads per (decode token, head).
+// Merges a decode token's key ranges.  One block of DH threads per (decode token, head): the threads first
+// share the ranges among themselves for the maximum and the sum (so that the loads of different ranges
+// are in flight together), then each thread adds up its element over the ranges in order.
 __global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, const float* __restrict__ ws_o,
                                               bf16_t* __restrict__ out, const int* __restrict__ positions,
                                               const int* __restrict__ dec_tokens, int max_splits, int kSplit,
                                               int ret_mode, int ret_param, int Hq, int Hkv, int DH, int cols) {
+  __shared__ float red_max[4], red_sum[4];
+  __shared__ int red_nan[4];
   const int d = blockIdx.x / Hq, h = blockIdx.x % Hq;
   const int n = dec_tokens[d];
   const int pos = positions[n];
@@ -518,20 +629,49 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, c
   const int ns = pos / kSplit - first / kSplit + 1;
   const int G = Hq / Hkv, hk = h / G, c = h - hk * G;
   const size_t item0 = ((size_t)d * Hkv + hk) * max_splits;
+  const float* ml = ws_ml + (item0 * cols + c) * 2;  // range s: + s * cols * 2
+  const float* wo = ws_o + (item0 * cols + c) * DH;  // range s: + s * cols * DH
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = (blockDim.x + 63) >> 6;
+
   float mx = -INFINITY;
-  for (int s = 0; s < ns; ++s) mx = fmaxf(mx, ws_ml[((item0 + s) * cols + c) * 2]);  // NaN (a missing page) stays
-  bool nan = false;
-  float l = 0.f;
-  for (int s = 0; s < ns; ++s) {
-    const float ms = ws_ml[((item0 + s) * cols + c) * 2];
-    nan = nan || ms != ms;
-    if (ms != -INFINITY && ms == ms) l += ws_ml[((item0 + s) * cols + c) * 2 + 1] * exp2f(ms - mx);
+  int nan = 0;
+  for (int s = threadIdx.x; s < ns; s += blockDim.x) {
+    const float ms = ml[(size_t)s * cols * 2];
+    nan |= ms != ms;  // a missing page
+    mx = fmaxf(mx, ms);
   }
+  mx = wave_max(mx);
+  nan = __any(nan);
+  if (lane == 0) {
+    red_max[wave] = mx;
+    red_nan[wave] = nan;
+  }
+  __syncthreads();
+  mx = red_max[0];
+  nan = red_nan[0];
+  for (int w = 1; w < waves; ++w) {
+    mx = fmaxf(mx, red_max[w]);
+    nan |= red_nan[w];
+  }
+  float l = 0.f;
+  for (int s = threadIdx.x; s < ns; s += blockDim.x) {
+    const float ms = ml[(size_t)s * cols * 2];
+    const float ls = ml[(size_t)s * cols * 2 + 1];
+    if (ms != -INFINITY && ms == ms) l += ls * exp2f(ms - mx);
+  }
+  l = wave_sum(l);
+  if (lane == 0) red_sum[wave] = l;
+  __syncthreads();
+  l = red_sum[0];
+  for (int w = 1; w < waves; ++w) l += red_sum[w];
+
   for (int e = threadIdx.x; e < DH; e += blockDim.x) {
     float o = 0.f;
+#pragma unroll 8
     for (int s = 0; s < ns; ++s) {
-      const float ms = ws_ml[((item0 + s) * cols + c) * 2];
-      if (ms != -INFINITY && ms == ms) o += ws_o[((item0 + s) * cols + c) * DH + e] * exp2f(ms - mx);
+      const float ms = ml[(size_t)s * cols * 2];
+      const float v = wo[(size_t)s * cols * DH + e];
+      o += (ms != -INFINITY && ms == ms) ? v * exp2f(ms - mx) : 0.f;
     }
     const float r = nan ? __builtin_nanf("") : (l > 0.f ? o / l : 0.f);
     out[((size_t)n * Hq + h) * DH + e] = float_to_bf16(r);

@@ -22,12 +22,15 @@ typedef uint16_t bf16_t;  // raw bits of a bfloat16
 
 __device__ __forceinline__ float bf16_to_float(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// round to nearest even, NaN stays NaN
-__device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  uint32_t x = __float_as_uint(f);
-  if ((x & 0x7fffffffu) > 0x7f800000u) return (bf16_t)0x7fc0;
-  x += 0x7fffu + ((x >> 16) & 1u);
-  return (bf16_t)(x >> 16);
+// round to nearest even (NaN stays NaN), by the hardware's conversion
+__device__ __forceinline__ bf16_t float_to_bf16(float f) { return __builtin_bit_cast(bf16_t, (__bf16)f); }
+
+// two values into one word (lo in the low half), one conversion instruction
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 template <typename T>

@@ -38,8 +38,8 @@ __device__ __forceinline__ void store4<float>(float* p, float a, float b, float 
 }
 template <>
 __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, float b, float c, float d, bool vec) {
-  const uint32_t lo = (uint32_t)float_to_bf16(a) | ((uint32_t)float_to_bf16(b) << 16);
-  const uint32_t hi = (uint32_t)float_to_bf16(c) | ((uint32_t)float_to_bf16(d) << 16);
+  const uint32_t lo = pack_bf16(a, b);
+  const uint32_t hi = pack_bf16(c, d);
   if (vec) {
     *reinterpret_cast<uint2*>(p) = uint2{lo, hi};
   } else {

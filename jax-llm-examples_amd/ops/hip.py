@@ -285,7 +285,7 @@ class HipOps:
                    n, hq, hk, dh, max(ps, 1), 0 if kv_cache is None else 1)
         return q
 
-    PREFILL_TILE = int(__import__("os").environ.get("JLE_PREFILL_TILE", "32"))  # tokens per prefill work item
+    PREFILL_TILE = 32  # tokens per prefill work item (the kernels take 16 or 32)
     DECODE_ITEMS = 1024  # decode attention: work items (wavefronts) to aim for
 
     def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1):
