@@ -36,6 +36,7 @@ _SIGNATURES = {
                              _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
 
@@ -70,6 +71,7 @@ def load_library():
             fn.argtypes = args
             fn.restype = ctypes.c_int
         lib.jle_attention_mfma_supported.argtypes = [_i, _i, _i, _i]  # a query, not a launch: no stream
+        lib.jle_gemm_stream_supported.argtypes = [_i, _i, _i]
         lib._jle_path = path
         _LIB = lib
     return _LIB
@@ -244,6 +246,34 @@ class HipOps:
                    int(out_f32), m, nout, k, g, int(tiled))
         return out
 
+    STREAM_MAX_ROWS = 160  # rows per group, on average, up to which the weight-streaming grouped product is used
+
+    def stream_supported(self, nout: int, k: int, swiglu: bool) -> bool:
+        return bool(self.lib.jle_gemm_stream_supported(nout, k, int(swiglu)))
+
+    def gemm_stream(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
+                    waves: int = 0):
+        """bfloat16 product on MFMA for about a hundred rows per group, weights in the streaming layout and
+        read once per 192 rows of a group (see ``gemm_stream.hip``)."""
+        if b.dim() == 2:
+            b = b.unsqueeze(0)
+        g, nout, k = b.shape
+        m = rows if rows is not None else (a_rows.numel() if a_rows is not None else a.shape[0])
+        self._chk(a, torch.bfloat16, None, "A")
+        self._chk(b, torch.bfloat16, None, "B")
+        if a.shape[1] != k:
+            raise KernelError(f"inner sizes differ: A {tuple(a.shape)}, B {tuple(b.shape)}")
+        if a.numel() >= 2 ** 32:
+            raise KernelError("the weight-streaming grouped product addresses its rows with 32 bits")
+        if not self.stream_supported(nout, k, swiglu):
+            raise KernelError(f"the weight-streaming grouped product needs an inner size that is a multiple of 256 and "
+                              f"whole tiles of 16 weight rows (32 with the fused activation), got {nout} x {k}")
+        out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
+                          device=a.device)
+        self._call("jle_gemm_stream", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
+                   int(out_f32), m, nout, k, g, m, int(waves))
+        return out
+
     def lm_head(self, h, w, tiled: bool = False):
         """float32 logits; ``tiled``: ``w`` is in the streaming layout (``ops/layout.py``)."""
         if h.dtype == torch.float32:
@@ -403,6 +433,11 @@ class HipOps:
             act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,
                                    tiled=tiled)
             routed = self.gemm_skinny(act, w_down, offsets=offsets, tiled=tiled)
+        elif (mfma and tiled and n * k <= self.STREAM_MAX_ROWS * e and self.stream_supported(f2, d, True)
+              and self.stream_supported(d, f2 // 2, False)):
+            # around a hundred rows per expert: still bound by reading the weights, which this kernel reads once
+            act = self.gemm_stream(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True)
+            routed = self.gemm_stream(act, w_down, offsets=offsets)
         elif mfma:
             act = self.gemm_grouped(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,
                                     tiled=tiled)
