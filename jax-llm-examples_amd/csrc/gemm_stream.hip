@@ -11,14 +11,13 @@
 // and are used once; the rows of X are what the wavefronts of a block share, through shared memory, 64 k
 // at a time, laid out as the B operands are read (with the 16 rows of a piece swizzled so that neither
 // writing nor reading collides).  A stage's weights are asked for four stages ahead (they come from memory,
-// and every wavefront of the block waits for the slowest at every stage), its rows two stages ahead (they come
-// from the cache after the first block that used them).  K must be a multiple of 256: whole rounds of four.
-// Groups with more than 192 rows are done in passes (each reads the weights again).
+// and every wavefront of the block waits for the slowest at every stage), its rows two stages ahead (they
+// come from the cache after the first block that used them).  K must be a multiple of 256: whole rounds of
+// four stages.  Groups with more than 192 rows are done in passes (each reads the weights again).
 //
-// Work items are (group, pass, block of WAVES * 32 weight rows), the last fastest.  The hardware deals
-// consecutive blocks of the grid to the 8 dies in turn; the kernel undoes that, so that each die works on a
-// contiguous stretch of items: the blocks that share a group's rows of X then run on the same die, next to
-// the same cache, at the same time.  Items without rows leave at once.
+// Work items are (group, pass, block of WAVES * 32 weight rows), the last fastest, so the blocks of a group
+// are dealt to all dies in turn and a group with many rows slows all of them alike.  Items without rows
+// leave at once.
 #include "common.h"
 
 using namespace jle;
@@ -61,7 +60,7 @@ __device__ __forceinline__ void stream_block(const bf16_t* __restrict__ X, const
   constexpr int CPT = (CHUNKS + THREADS - 1) / THREADS;  // per thread
   const int lane = threadIdx.x & 63;
   const int r = lane & 15, g = lane >> 4;
-  const int nstage = K / BK;  // a multiple of WAHEAD
+  const int nstage = K / BK;  // a multiple of 4
   const int half = Nout >> 1;
 
   // who brings which pieces of X: piece c is 8 k of row c / 8, 8 consecutive threads a row's 128 bytes
@@ -183,11 +182,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* _
                                                                  const int* __restrict__ offsets,
                                                                  const int* __restrict__ a_rows,
                                                                  const float* __restrict__ scale, int M, int Nout,
-                                                                 int K, int nblk, int passes, int items) {
+                                                                 int K, int nblk, int passes) {
   __shared__ __attribute__((aligned(16))) bf16_t sX[2][kRows * BK];
-  const int per_die = (items + 7) >> 3;
-  const int item = (blockIdx.x & 7) * per_die + (blockIdx.x >> 3);
-  if (item >= items) return;
+  const int item = blockIdx.x;
   const int nb = item % nblk, pass = (item / nblk) % passes, e = item / (nblk * passes);
   int row_lo = 0, row_hi = M;
   if (offsets != nullptr) {
@@ -230,10 +227,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* _
 template <bool SW, typename OT, int WV>
 void launch_stream(int nblk, int passes, int G, hipStream_t s, const void* X, const void* W, void* Y,
                    const int* offsets, const int* a_rows, const float* scale, int M, int Nout, int K) {
-  const int items = nblk * passes * G;
-  const int per_die = (items + 7) / 8;
-  hipLaunchKernelGGL((gemm_stream_kernel<SW, OT, WV>), dim3(per_die * 8), dim3(WV * 64), 0, s, (const bf16_t*)X,
-                     (const bf16_t*)W, (OT*)Y, offsets, a_rows, scale, M, Nout, K, nblk, passes, items);
+  hipLaunchKernelGGL((gemm_stream_kernel<SW, OT, WV>), dim3(nblk * passes * G), dim3(WV * 64), 0, s,
+                     (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, offsets, a_rows, scale, M, Nout, K, nblk, passes);
 }
 
 }  // namespace

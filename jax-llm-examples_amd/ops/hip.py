@@ -436,6 +436,7 @@ class HipOps:
         elif (mfma and tiled and n * k <= self.STREAM_MAX_ROWS * e and self.stream_supported(f2, d, True)
               and self.stream_supported(d, f2 // 2, False)):
             # around a hundred rows per expert: still bound by reading the weights, which this kernel reads once
+            # per 192 rows of an expert
             act = self.gemm_stream(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True)
             routed = self.gemm_stream(act, w_down, offsets=offsets)
         elif mfma:
