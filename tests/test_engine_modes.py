@@ -15,15 +15,16 @@ import torch
 import traces
 from jax_llm_examples_amd.engine.replay import make_runner
 from plain_llama4 import PlainModel
-from tiny_configs import TINY
+from tiny_configs import FAST, TINY, write_tiny
 
-LENGTHS = {"A": [1, 80, 33, 47, 64, 9], "B": [120, 2, 49, 96, 31, 77], "C": [61, 40, 5, 83], "D": [37, 70, 3, 55, 64, 21]}
+LENGTHS = {"A": [1, 80, 33, 47, 64, 9], "B": [120, 2, 49, 96, 31, 77], "C": [61, 40, 5, 83], "D": [37, 70, 3, 55, 64, 21],
+           "F": [300, 40, 170, 33]}
 MODES = {"whole": traces.whole, "tail": traces.tail, "portions": traces.portions, "mixed": traces.mixed}
 TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}  # of the largest logit of the request
 
 
 def _vocab(name):
-    c = TINY[name]
+    c = {**TINY, **FAST}[name]
     return c.get("text_config", c)["vocab_size"]
 
 
@@ -74,6 +75,30 @@ def test_gpu_float32(model_dirs, name, mode):
 @pytest.mark.parametrize("name", list(TINY))
 def test_gpu_bfloat16(model_dirs_bf16, name, mode):
     _check(name, model_dirs_bf16[name], "bfloat16", "cuda:0", mode, reference_ops=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+def test_gpu_bfloat16_sizes_of_the_fast_kernels(tmp_path_factory, mode, monkeypatch):
+    """The tiny configurations are too small for the kernels that serving sizes get (keys shared between the
+    query heads of a kv head, expert matrices in the streaming layout, the weight-streaming grouped product
+    in prefill): this one is not."""
+    folder = write_tiny("F", str(tmp_path_factory.mktemp("models_fast") / "F"), torch.bfloat16)
+    runner = make_runner(folder, "bfloat16", 1024, "cuda:0")
+    moe = [b.feed_forward for b in runner.model.blocks]
+    assert all(ff.tiled for ff in moe), "the expert matrices of this configuration fit the streaming layout"
+    from jax_llm_examples_amd.ops.hip import HipOps
+    calls = {"stream": 0}
+    inner = HipOps.gemm_stream
+
+    def counted(self, *a, **kw):
+        calls["stream"] += 1
+        return inner(self, *a, **kw)
+
+    monkeypatch.setattr(HipOps, "gemm_stream", counted)
+    _check("F", folder, "bfloat16", "cuda:0", mode, reference_ops=False)
+    if mode in ("whole", "tail"):  # the other modes cut the prompts into portions too short for it
+        assert calls["stream"] > 0, "no step went through the weight-streaming grouped product"
 
 
 @pytest.mark.gpu

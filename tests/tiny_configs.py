@@ -55,9 +55,25 @@ TINY = {
     },
 }
 
+# Small, but with the sizes that the fast kernels need (GPU tests only): head size 128 with five query heads per
+# kv head (prefill attention shares keys between them), widths that are multiples of 256 (the expert matrices go
+# into the streaming layout and prefill goes through the weight-streaming grouped product)
+FAST = {
+    "F": {
+        "architectures": ["Llama4ForCausalLM"],
+        "seed": 53,
+        "num_hidden_layers": 2, "hidden_size": 256, "num_attention_heads": 10, "num_key_value_heads": 2,
+        "head_dim": 128, "interleave_moe_layer_step": 1, "num_local_experts": 4, "num_experts_per_tok": 1,
+        "intermediate_size": 256, "intermediate_size_mlp": 512, "vocab_size": 600, "rope_theta": 10000.0,
+        "rope_scaling": None, "no_rope_layers": [1, 0], "attention_chunk_size": 96, "use_qk_norm": True,
+        "attn_temperature_tuning": True, "floor_scale": 64, "attn_scale": 0.1, "rms_norm_eps": 1e-5,
+        "tie_word_embeddings": False,
+    },
+}
+
 
 def tiny_config_json(name: str) -> dict:
-    c = {k: v for k, v in TINY[name].items() if k != "seed"}
+    c = {k: v for k, v in {**TINY, **FAST}[name].items() if k != "seed"}
     return c
 
 
@@ -68,4 +84,5 @@ def write_tiny(name: str, out_dir: str, dtype=torch.float32) -> str:
     top = tiny_config_json(name)
     arch = get_architecture(top["architectures"][0])
     cfg = arch.parse_config(top)
-    return write_random_model(arch, cfg, out_dir, TINY[name]["seed"], dtype, architecture=top["architectures"][0])
+    return write_random_model(arch, cfg, out_dir, {**TINY, **FAST}[name]["seed"], dtype,
+                              architecture=top["architectures"][0])
