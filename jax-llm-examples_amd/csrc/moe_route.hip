@@ -6,49 +6,64 @@ using namespace jle;
 
 constexpr int kMaxTopK = 8;
 
-// Router logits: logits[n, e] = sum_d h[n, d] * W[e, d], float32.  One wavefront per expert and
+// Router logits: logits[n, e] = sum_d h[n, d] * W[e, d], float32.  One wavefront per EPW experts and
 // TPB tokens; a lane adds the terms of its float4 chunks (chunk = lane, lane + 64, ...) in
-// order, then the lanes' sums are added by a butterfly: the order is the same for any TPB.
-template <int TPB, bool VEC>
+// order, then the lanes' sums are added by a butterfly: the order, and so the result, is the same for
+// any TPB and EPW (a token's expert choice must not depend on what else is in the step).
+template <int TPB, int EPW, bool VEC>
 __global__ __launch_bounds__(256) void moe_logits_kernel(const float* __restrict__ h, const float* __restrict__ w,
                                                          float* __restrict__ logits, int N, int D, int E) {
   const int lane = threadIdx.x & 63;
-  const int e = blockIdx.y * 4 + (threadIdx.x >> 6);
+  const int e0 = (blockIdx.y * 4 + (threadIdx.x >> 6)) * EPW;
   const int n0 = blockIdx.x * TPB;
-  if (e >= E) return;
-  const float* we = w + (size_t)e * D;
-  float acc[TPB];
+  if (e0 >= E) return;
+  const float* we[EPW];
 #pragma unroll
-  for (int t = 0; t < TPB; ++t) acc[t] = 0.f;
+  for (int j = 0; j < EPW; ++j) we[j] = w + (size_t)min(e0 + j, E - 1) * D;  // past the last: computed, not stored
+  float acc[TPB][EPW];
+#pragma unroll
+  for (int t = 0; t < TPB; ++t)
+#pragma unroll
+    for (int j = 0; j < EPW; ++j) acc[t][j] = 0.f;
   if (VEC) {  // D is a multiple of 4: rows are 16-byte aligned
     const int D4 = D >> 2;
-#pragma unroll 4
+#pragma unroll 2
     for (int c = lane; c < D4; c += 64) {
-      const float4 wv = *reinterpret_cast<const float4*>(we + 4 * c);
+      float4 wv[EPW];
+#pragma unroll
+      for (int j = 0; j < EPW; ++j) wv[j] = *reinterpret_cast<const float4*>(we[j] + 4 * c);
 #pragma unroll
       for (int t = 0; t < TPB; ++t) {
         if (n0 + t < N) {
           const float4 xv = *reinterpret_cast<const float4*>(h + (size_t)(n0 + t) * D + 4 * c);
-          acc[t] += xv.x * wv.x;
-          acc[t] += xv.y * wv.y;
-          acc[t] += xv.z * wv.z;
-          acc[t] += xv.w * wv.w;
+#pragma unroll
+          for (int j = 0; j < EPW; ++j) {
+            acc[t][j] += xv.x * wv[j].x;
+            acc[t][j] += xv.y * wv[j].y;
+            acc[t][j] += xv.z * wv[j].z;
+            acc[t][j] += xv.w * wv[j].w;
+          }
         }
       }
     }
   } else {
     for (int d = lane; d < D; d += 64) {
-      const float wv = we[d];
 #pragma unroll
       for (int t = 0; t < TPB; ++t)
-        if (n0 + t < N) acc[t] += h[(size_t)(n0 + t) * D + d] * wv;
+        if (n0 + t < N) {
+          const float xv = h[(size_t)(n0 + t) * D + d];
+#pragma unroll
+          for (int j = 0; j < EPW; ++j) acc[t][j] += xv * we[j][d];
+        }
     }
   }
 #pragma unroll
-  for (int t = 0; t < TPB; ++t) {
-    const float v = wave_sum(acc[t]);
-    if (lane == 0 && n0 + t < N) logits[(size_t)(n0 + t) * E + e] = v;
-  }
+  for (int t = 0; t < TPB; ++t)
+#pragma unroll
+    for (int j = 0; j < EPW; ++j) {
+      const float v = wave_sum(acc[t][j]);
+      if (lane == 0 && n0 + t < N && e0 + j < E) logits[(size_t)(n0 + t) * E + e0 + j] = v;
+    }
 }
 
 // The k largest logits of each token (lowest index first among equals) and their sigmoids.
@@ -97,14 +112,18 @@ JLE_API int jle_moe_route(const float* h, const float* w, int* ids, float* gates
   if (N <= 0) return 0;
   if (k < 1 || k > kMaxTopK || k > E || E > 4096 || logits == nullptr) return JLE_BAD_ARG;
   const bool vec = D % 4 == 0 && (((uintptr_t)h | (uintptr_t)w) & 15) == 0;
-  const bool many = N >= 512;  // fewer rows: a block per token keeps more blocks in flight
-  dim3 g(many ? (N + 7) / 8 : N, (E + 3) / 4), b(256);
+  // few rows: a wavefront per (token, expert) keeps more of them in flight; many: a wavefront takes 2 tokens
+  // and 4 experts, so that the rows of h are read 4 times less often
+  const bool many = N >= 512;
+  dim3 b(256);
   if (many) {
-    if (vec) hipLaunchKernelGGL((moe_logits_kernel<8, true>), g, b, 0, s, h, w, logits, N, D, E);
-    else hipLaunchKernelGGL((moe_logits_kernel<8, false>), g, b, 0, s, h, w, logits, N, D, E);
+    dim3 g((N + 1) / 2, (E + 15) / 16);
+    if (vec) hipLaunchKernelGGL((moe_logits_kernel<2, 4, true>), g, b, 0, s, h, w, logits, N, D, E);
+    else hipLaunchKernelGGL((moe_logits_kernel<2, 4, false>), g, b, 0, s, h, w, logits, N, D, E);
   } else {
-    if (vec) hipLaunchKernelGGL((moe_logits_kernel<1, true>), g, b, 0, s, h, w, logits, N, D, E);
-    else hipLaunchKernelGGL((moe_logits_kernel<1, false>), g, b, 0, s, h, w, logits, N, D, E);
+    dim3 g(N, (E + 3) / 4);
+    if (vec) hipLaunchKernelGGL((moe_logits_kernel<1, 1, true>), g, b, 0, s, h, w, logits, N, D, E);
+    else hipLaunchKernelGGL((moe_logits_kernel<1, 1, false>), g, b, 0, s, h, w, logits, N, D, E);
   }
   JLE_LAUNCH_CHECK();
   hipLaunchKernelGGL(moe_topk_kernel, dim3((N + 127) / 128), dim3(128), 0, s, logits, ids, gates, N, E, k);

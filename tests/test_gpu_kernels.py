@@ -239,6 +239,18 @@ def test_moe_route(ops, ref, n, d, e, k):
     assert torch.equal(ids, rid) and torch.allclose(gates, rg, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("n,d,e,k", [(700, 320, 16, 1), (600, 90, 6, 2), (520, 64, 37, 3)])
+def test_router_logits_of_a_token_do_not_depend_on_the_batch(ops, n, d, e, k):
+    """Many rows take another kernel shape than few; the sums must come out bit for bit the same, or a token's
+    experts would depend on what else is in the step."""
+    h, w = _rand(n, d, seed=1), _rand(e, d, scale=0.05, seed=2)
+    ids, gates, logits = ops.moe_route(h, w, k, want_logits=True)
+    assert torch.allclose(logits, h @ w.t(), rtol=1e-4, atol=1e-5)
+    for lo, hi in [(0, 1), (n - 1, n), (100, 107), (3, 300)]:
+        i2, g2, l2 = ops.moe_route(h[lo:hi].contiguous(), w, k, want_logits=True)
+        assert torch.equal(l2, logits[lo:hi]) and torch.equal(i2, ids[lo:hi]) and torch.equal(g2, gates[lo:hi])
+
+
 def test_moe_route_lowest_index_wins_ties(ops):
     h = _rand(5, 64, seed=1)
     w = _rand(1, 64, seed=2).expand(6, 64).contiguous()  # every expert the same score
