@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void paged_attention_generic_kernel(
     const int* __restrict__ token_segment, const int* __restrict__ block_table, int table_width, int ret_mode,
     int ret_param, float scale, int N, int Hq, int Hkv, int dh, int ps) {
   const int lane = threadIdx.x & 63;
-  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int item = blockIdx.x * 4 + wave_index();
   if (item >= N * Hq) return;  // whole wavefront leaves; no block-wide barrier below
   const int n = item / Hq, h = item - n * Hq;
   const int hk = h / (Hq / Hkv);

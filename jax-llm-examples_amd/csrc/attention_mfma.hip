@@ -33,6 +33,7 @@ using namespace jle;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;  // (register arrays of HIP's uint4 may end up in scratch)
 
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -75,9 +76,9 @@ __device__ __forceinline__ float column_sum(float v) {
 //   st[ct][tt]: scores of key tile tt (keys kb + 16 tt + 4 g + i in element i); act0 / act1: the tile exists
 //   vraw[dt]: for element row 16 dt + (lane % 16): keys 4 g .. 4 g + 3 of tile 0 (x, y) and of tile 1 (z, w)
 //   l: each lane's own part of the column's sum (column_sum at the end gives the whole)
-template <int DH, int CT, bool MASKED>
+template <int DH, int CT, bool MASKED, typename V4>
 __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], bool act0, bool act1,
-                                                   const uint4 (&vraw)[DH / 16], int kb, const Columns (&col)[CT],
+                                                   const V4 (&vraw)[DH / 16], int kb, const Columns (&col)[CT],
                                                    int k_lo, int k_hi, float scale_log2, float (&m)[CT],
                                                    float (&l)[CT], f32x4 (&acc)[CT][DH / 16]) {
   constexpr int DT = DH / 16;
@@ -146,7 +147,7 @@ __device__ __forceinline__ void softmax_and_values(const f32x4 (&st)[CT][2], boo
     }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      uint4 vv = vraw[dt];
+      V4 vv = vraw[dt];
       vv.x &= keep[0][0];
       vv.y &= keep[0][1];
       vv.z &= keep[1][0];
@@ -216,61 +217,81 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
     for (int dt = 0; dt < DT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // The keys of a step are asked for one step ahead (they are in registers when the step begins); its
-  // values are asked for at its beginning and arrive while the scores are worked on.
-  uint4 kraw[2][KC];
-  const bf16_t* vbase[2];
+  // The keys and values of a step are asked for one step ahead: they are in registers when the step begins.
+  // Their pages are looked up one step before that, through the scalar path (everything about the cursor is
+  // the same in all lanes), so a step never waits for the block table and then again for the data.
+  u32x4 kraw[2][KC], vnext[DT];
   bool active[2];
-  auto locate_and_load_keys = [&](int kb) {
+  const int kb_first = (k_lo / 32) * 32;
+  int next_kb = kb_first;                                   // the cursor: the next step to ask for
+  int page_index = next_kb / ps, page_off = next_kb % ps;  // of its first key
+  int pages[2], offs[2];                                    // per key tile: page (-1: none) and first key within it
+  auto look_up = [&]() {
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      const int key0 = kb + 16 * tt;
-      active[tt] = key0 <= k_hi && key0 + 15 >= k_lo;
-      int page = -1;
-      if (active[tt]) {
-        page = table[key0 / ps];
-        if (page < 0) {
-          bad = true;
-          active[tt] = false;
-        }
+      const int key0 = next_kb + 16 * tt;
+      int idx = page_index, off = page_off + 16 * tt;
+      if (off >= ps) {
+        off -= ps;
+        ++idx;
       }
-      vbase[tt] = nullptr;
-#pragma unroll
-      for (int c = 0; c < KC; ++c) kraw[tt][c] = uint4{0u, 0u, 0u, 0u};
-      if (active[tt]) {
-        const bf16_t* kbase = kv + (size_t)page * page_stride + (size_t)hk * plane;
-        const int off = key0 % ps;
-        const bf16_t* krow = kbase + (size_t)(off + c16) * DH + g * 8;
-        vbase[tt] = kbase + (size_t)Hkv * plane + off + 4 * g;  // + d * ps
-#pragma unroll
-        for (int c = 0; c < KC; ++c) kraw[tt][c] = *reinterpret_cast<const uint4*>(krow + c * 32);
+      offs[tt] = off;
+      pages[tt] = -1;
+      if (key0 <= k_hi && key0 + 15 >= k_lo) {
+        pages[tt] = table[idx];
+        if (pages[tt] < 0) bad = true;  // the tile is then left out, and the result is NaN
       }
     }
   };
+  auto load_step = [&]() {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vnext[dt] = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      active[tt] = pages[tt] >= 0;
+#pragma unroll
+      for (int c = 0; c < KC; ++c) kraw[tt][c] = u32x4{0u, 0u, 0u, 0u};
+      if (active[tt]) {
+        const bf16_t* kbase = kv + (size_t)pages[tt] * page_stride + (size_t)hk * plane;
+        const bf16_t* krow = kbase + (size_t)(offs[tt] + c16) * DH + g * 8;
+        const bf16_t* vcol = kbase + (size_t)Hkv * plane + offs[tt] + 4 * g;  // + d * ps
+#pragma unroll
+        for (int c = 0; c < KC; ++c) kraw[tt][c] = *reinterpret_cast<const u32x4*>(krow + c * 32);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const uint2 t = *reinterpret_cast<const uint2*>(vcol + (size_t)(dt * 16 + c16) * ps);
+          if (tt == 0) {
+            vnext[dt].x = t.x;
+            vnext[dt].y = t.y;
+          } else {
+            vnext[dt].z = t.x;
+            vnext[dt].w = t.y;
+          }
+        }
+      }
+    }
+    next_kb += 32;
+    page_off += 32;  // a page holds at least 16 keys: at most two pages further
+    if (page_off >= ps) {
+      page_off -= ps;
+      ++page_index;
+    }
+    if (page_off >= ps) {
+      page_off -= ps;
+      ++page_index;
+    }
+    look_up();
+  };
   int all_lo, all_hi;
   common_range<CT>(col, all_lo, all_hi);
-  const int kb_first = (k_lo / 32) * 32;
-  if (kb_first <= k_hi) locate_and_load_keys(kb_first);
+  look_up();
+  if (kb_first <= k_hi) load_step();
   for (int kb = kb_first; kb <= k_hi; kb += 32) {
     f32x4 st[CT][2];
     const bool act0 = active[0], act1 = active[1];
-    // this step's values
-    uint4 vraw[DT];
+    u32x4 vraw[DT];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      vraw[dt] = uint4{0u, 0u, 0u, 0u};
-      const size_t drow = (size_t)(dt * 16 + c16) * ps;
-      if (act0) {
-        const uint2 t0 = *reinterpret_cast<const uint2*>(vbase[0] + drow);
-        vraw[dt].x = t0.x;
-        vraw[dt].y = t0.y;
-      }
-      if (act1) {
-        const uint2 t1 = *reinterpret_cast<const uint2*>(vbase[1] + drow);
-        vraw[dt].z = t1.x;
-        vraw[dt].w = t1.y;
-      }
-    }
+    for (int dt = 0; dt < DT; ++dt) vraw[dt] = vnext[dt];
     // scores from the keys that are already here
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
@@ -284,8 +305,8 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
           st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
       }
     }
-    // the next step's keys (overwrites kraw, vbase and active: this step keeps act0 / act1 and vraw)
-    if (kb + 32 <= k_hi) locate_and_load_keys(kb + 32);
+    // the next step's keys and values (this step keeps act0 / act1 and vraw)
+    if (kb + 32 <= k_hi) load_step();
     if (__all(act0 && act1 && kb >= all_lo && kb + 31 <= all_hi))
       softmax_and_values<DH, CT, false>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
     else
@@ -298,14 +319,15 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
 // ------------------------------------------------------------------ prefill portions
 // tiles: [num_tiles][2] = (first token, number of tokens <= 16 * CT), all of one segment.
 // One wavefront per (tile, query head); the heads of one kv head are neighbours.
+// (launch bounds: with one column tile and head sizes up to 128 the registers are held to what lets two wavefronts share a SIMD)
 template <int DH, int CT>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(
+__global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ tiles, int num_tiles, int ret_mode, int ret_param, float scale_log2,
     int Hq, int Hkv, int ps) {
   const int lane = threadIdx.x & 63;
-  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int item = blockIdx.x * 4 + wave_index();
   if (item >= num_tiles * Hq) return;
   // the last tiles of a segment have the most keys: they are started first
   const int tile = num_tiles - 1 - item / Hq, h = item % Hq;
@@ -365,7 +387,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
   constexpr int CPT = (NCH + THREADS - 1) / THREADS;  // per thread
   constexpr int SK = 32 * KP, SV = 2 * DH * 16;       // elements of a buffer: keys, then values
   __shared__ __attribute__((aligned(16))) bf16_t smem[2][SK + SV];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = wave_index();
   const int c16 = lane & 15, g = lane >> 4;
   const int G = Hq / Hkv;
   const int hchunks = (G + WAVES - 1) / WAVES;
@@ -563,13 +585,13 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
 // (decode token, kv head, key range); ws_ml: [item][16 * CT][2], ws_o: [item][16 * CT][DH],
 // item = (d * Hkv + hk) * max_splits + split.
 template <int DH, int CT>
-__global__ __launch_bounds__(256) void attention_decode_kernel(
+__global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, float* __restrict__ ws_ml, float* __restrict__ ws_o,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ dec_tokens, int num_dec, int max_splits, int kSplit, int ret_mode,
     int ret_param, float scale_log2, int Hq, int Hkv, int ps) {
   const int lane = threadIdx.x & 63;
-  const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int item = blockIdx.x * 4 + wave_index();
   if (item >= num_dec * Hkv * max_splits) return;
   const int split = item % max_splits;
   const int hk = (item / max_splits) % Hkv;
@@ -631,7 +653,7 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, c
   const size_t item0 = ((size_t)d * Hkv + hk) * max_splits;
   const float* ml = ws_ml + (item0 * cols + c) * 2;  // range s: + s * cols * 2
   const float* wo = ws_o + (item0 * cols + c) * DH;  // range s: + s * cols * DH
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = (blockDim.x + 63) >> 6;
+  const int lane = threadIdx.x & 63, wave = wave_index(), waves = (blockDim.x + 63) >> 6;
 
   float mx = -INFINITY;
   int nan = 0;

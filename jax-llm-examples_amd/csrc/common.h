@@ -48,6 +48,10 @@ struct Num<bf16_t> {
   static __device__ __forceinline__ float round(float v) { return bf16_to_float(float_to_bf16(v)); }
 };
 
+// The wavefront's index within its block, as a value the compiler knows to be the same in all lanes (so what
+// is computed from it stays in scalar registers and uniform loads take the scalar path).
+__device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

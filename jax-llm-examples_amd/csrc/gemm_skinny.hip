@@ -54,7 +54,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   }
   const int tok0 = row_lo + blockIdx.y * (16 * MT);
   if (tok0 >= row_hi) return;  // the whole block
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = wave_index();
   const int r = lane & 15, g = lane >> 4;
   const bf16_t* We = W + (size_t)e * Nout * K;
   const int half = Nout >> 1;

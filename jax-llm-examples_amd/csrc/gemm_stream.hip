@@ -195,7 +195,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* _
   if (tok0 >= row_hi) return;  // the whole block
   const int live = min(kRows, row_hi - tok0);  // rows of this pass
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = wave_index();
   const int nkb = K >> 5;
   const int half = Nout >> 1;
   const bf16_t* We = W + (size_t)e * Nout * K;

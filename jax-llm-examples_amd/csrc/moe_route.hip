@@ -14,7 +14,7 @@ template <int TPB, int EPW, bool VEC>
 __global__ __launch_bounds__(256) void moe_logits_kernel(const float* __restrict__ h, const float* __restrict__ w,
                                                          float* __restrict__ logits, int N, int D, int E) {
   const int lane = threadIdx.x & 63;
-  const int e0 = (blockIdx.y * 4 + (threadIdx.x >> 6)) * EPW;
+  const int e0 = (blockIdx.y * 4 + wave_index()) * EPW;
   const int n0 = blockIdx.x * TPB;
   if (e0 >= E) return;
   const float* we[EPW];
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
   }
   __syncthreads();
   for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = starts[e];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63, wave = wave_index(), waves = blockDim.x >> 6;
   for (int e = wave; e < E; e += waves) {
     if (counts[e] == 0) continue;
     int run = starts[e];

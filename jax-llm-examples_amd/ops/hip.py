@@ -316,7 +316,10 @@ class HipOps:
         return q
 
     PREFILL_TILE = 32  # tokens per prefill work item (the kernels take 16 or 32)
-    DECODE_ITEMS = 1024  # decode attention: work items (wavefronts) to aim for
+    DECODE_ITEMS = 1024  # decode attention: work items (wavefronts) that run at once, one per SIMD
+    DECODE_MIN_SPLIT = 128  # keys per work item at least (fewer: the merge costs more than the spreading gains)
+    DECODE_FIT_SPLIT = 1024  # ... at most, to make the items fit in one go
+    DECODE_MAX_SPLIT = 512  # ... when there are more items than fit anyway
 
     def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1):
         """Work lists of the MFMA attention kernels for one step and one retention rule: the rows that are
@@ -334,11 +337,14 @@ class HipOps:
                 for t in range(0, n, self.PREFILL_TILE):
                     tiles += [o + t, min(self.PREFILL_TILE, n - t)]
             o += n
-        split, max_splits = 256, 1
+        split, max_splits = self.DECODE_MAX_SPLIT, 1
         if dec:
-            keys = sum(p - f + 1 for f, p in spans)
-            while split > 64 and keys * num_kv_heads // split < self.DECODE_ITEMS:
-                split //= 2
+            # the smallest range (a multiple of 32 keys) with which the work items still fit the GPU in one go:
+            # a compute unit that gets a second item beside its first takes much longer than the others
+            for cand in range(self.DECODE_MIN_SPLIT, self.DECODE_FIT_SPLIT + 1, 32):
+                if num_kv_heads * sum(p // cand - f // cand + 1 for f, p in spans) <= self.DECODE_ITEMS:
+                    split = cand
+                    break
             max_splits = max(p // split - f // split + 1 for f, p in spans)
         flat = torch.tensor(dec + tiles, dtype=torch.int32).to(device) if dec or tiles else None
         return {"num_dec": len(dec), "num_tiles": len(tiles) // 2, "max_splits": max_splits, "split": split,
