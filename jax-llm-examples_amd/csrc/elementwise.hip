@@ -201,14 +201,36 @@ __global__ void silu_mul_kernel(const T* __restrict__ in, T* __restrict__ out, i
   Num<T>::store(out + row * F + f, sg * u);
 }
 
+// bfloat16 rows whose halves are 16-byte aligned: 8 elements per thread
+__global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, int F) {
+  const size_t row = blockIdx.y;
+  const int f = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (f >= F) return;
+  const uint4 gv = *reinterpret_cast<const uint4*>(in + row * 2 * F + f);
+  const uint4 uv = *reinterpret_cast<const uint4*>(in + row * 2 * F + F + f);
+  const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+    const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+    o[i] = pack_bf16(g0 / (1.0f + expf(-g0)) * u0, g1 / (1.0f + expf(-g1)) * u1);
+  }
+  *reinterpret_cast<uint4*>(out + row * F + f) = uint4{o[0], o[1], o[2], o[3]};
+}
+
 JLE_API int jle_silu_mul(const void* in, void* out, int is_bf16, int N, int F, hipStream_t s) {
   if (N <= 0 || F <= 0) return 0;
   if (N > 65535 * 16) return JLE_BAD_ARG;
   dim3 g((F + 255) / 256, N), b(256);
-  if (is_bf16)
+  if (is_bf16 && F % 8 == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
+    dim3 g8((F / 8 + 255) / 256, N);
+    hipLaunchKernelGGL(silu_mul_bf16x8_kernel, g8, b, 0, s, (const bf16_t*)in, (bf16_t*)out, F);
+  } else if (is_bf16) {
     hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)in, (bf16_t*)out, F);
-  else
+  } else {
     hipLaunchKernelGGL(silu_mul_kernel<float>, g, b, 0, s, (const float*)in, (float*)out, F);
+  }
   JLE_LAUNCH_CHECK();
   return 0;
 }
