@@ -372,8 +372,7 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention
 // One block per (tile of up to 32 tokens, kv head, up to WAVES of its query heads): a wavefront per
 // query head.  The heads read the same keys and values, so every 32-key step is brought into shared
 // memory once by the whole block (the next step's data is in flight meanwhile) and each wavefront
-// takes its operands from there.  Keys get a row pitch of DH + 8 elements (16-byte reads of 16 rows then
-// hit all banks); values keep the page's layout [DH][16].
+// takes its operands from there (laid out so that no access meets another in a bank, see below).
 template <int DH, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
@@ -385,7 +384,13 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
   constexpr int THREADS = WAVES * 64;
   constexpr int NCH = 8 * DH;                         // 16-byte chunks per step: keys 2 x 16 x DH / 8, values the same
   constexpr int CPT = (NCH + THREADS - 1) / THREADS;  // per thread
-  constexpr int SK = 32 * KP, SV = 2 * DH * 16;       // elements of a buffer: keys, then values
+  // Shared memory of a buffer, in elements: keys, then values.  The placing is chosen so that neither the
+  // stores (neighbouring threads bring pieces of the two key tiles in turn) nor the loads meet in a bank:
+  //   keys:   tile tt, key row: tt * KT + row * KP (KP: 16 bytes more than a row; the second tile 64 bytes on)
+  //   values: tile tt, keys 4 g .. 4 g + 3 of element d: tt * VT + g * VP + d * 4 (what a lane loads as one
+  //           8-byte piece is laid out along d, so that 16 lanes read 128 contiguous bytes)
+  constexpr int KT = 16 * KP + 32, SK = 2 * KT;
+  constexpr int VP = DH * 4 + 16, VT = 4 * VP + 16, SV = 2 * VT;
   __shared__ __attribute__((aligned(16))) bf16_t smem[2][SK + SV];
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int c16 = lane & 15, g = lane >> 4;
@@ -446,21 +451,26 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
     const int c = threadIdx.x + THREADS * i;
     const int r = c >> 1;
     in_use[i] = c < NCH;
-    is_key[i] = r < 2 * DH;
-    if (is_key[i]) {
+    is_key[i] = r < 2 * DH || !in_use[i];  // (a chunk past the last reads the tile's first key again, for nothing)
+    if (!in_use[i]) {
+      src_off[i] = 0;
+      dst_off[i] = 0;
+    } else if (is_key[i]) {
       src_off[i] = (r / (DH / 8)) * DH + (r % (DH / 8)) * 8;
-      dst_off[i] = (my_tile * 16 + r / (DH / 8)) * KP + (r % (DH / 8)) * 8;
+      dst_off[i] = my_tile * KT + (r / (DH / 8)) * KP + (r % (DH / 8)) * 8;
     } else {
       const int r2 = r - 2 * DH;
       src_off[i] = (r2 >> 1) * ps + (r2 & 1) * 8;
-      dst_off[i] = SK + (my_tile * DH + (r2 >> 1)) * 16 + (r2 & 1) * 8;
+      dst_off[i] = SK + my_tile * VT + (2 * (r2 & 1)) * VP + (r2 >> 1) * 4;  // its second half: + VP
     }
   }
 
   bool bad = false;
-  // PF register sets: the data of the next PF steps are on their way while a step is worked on
+  // PF register sets: the data of the next PF steps are on their way while a step is worked on.  Every load
+  // is issued unconditionally (a tile that is not needed reads page 0, whose contents are then masked like any
+  // key out of range; a step past the last likewise), so that the wait for one set never includes the other.
   constexpr int PF = 2;
-  uint4 reg[PF][CPT];
+  u32x4 reg[PF][CPT];
   // The cursor: the next step to ask for (the same in all threads, so the block table is read through the
   // scalar path, which the wait for the bulk loads does not include).  The pages of a step are looked up
   // when the step before it is asked for.
@@ -481,23 +491,20 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
       pages[tt] = -1;
       if (key0 <= k_hi && key0 + 15 >= k_lo) {
         pages[tt] = table[idx];
-        if (pages[tt] < 0) bad = true;  // the tile is then read as zeros, and the block's result is NaN
+        if (pages[tt] < 0) bad = true;  // the block's result is NaN
       }
     }
   };
   look_up();
   auto load_step = [&](int set) {
-    const int page = my_tile ? pages[1] : pages[0];
+    const int page = max(my_tile ? pages[1] : pages[0], 0);
     const int off = my_tile ? offs[1] : offs[0];
-    const bf16_t* keys = kv + (size_t)(page < 0 ? 0 : page) * page_stride + (size_t)hk * plane;
+    const bf16_t* keys = kv + (size_t)page * page_stride + (size_t)hk * plane;
     const bf16_t* values = keys + (size_t)Hkv * plane + off;
     keys += (size_t)off * DH;
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      reg[set][i] = uint4{0u, 0u, 0u, 0u};
-      if (in_use[i] && page >= 0)
-        reg[set][i] = *reinterpret_cast<const uint4*>((is_key[i] ? keys : values) + src_off[i]);
-    }
+    for (int i = 0; i < CPT; ++i)
+      reg[set][i] = *reinterpret_cast<const u32x4*>((is_key[i] ? keys : values) + src_off[i]);
     next_kb += 32;
     page_off += 32;  // a page holds at least 16 keys: at most two pages further
     if (page_off >= ps) {
@@ -513,55 +520,60 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
   auto store_step = [&](int set, int buf) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i)
-      if (in_use[i]) *reinterpret_cast<uint4*>(&smem[buf][dst_off[i]]) = reg[set][i];
+      if (in_use[i]) {
+        if (is_key[i]) {
+          *reinterpret_cast<u32x4*>(&smem[buf][dst_off[i]]) = reg[set][i];
+        } else {  // 8 keys of one element: keys 0..3 to one lane group's place, 4..7 to the next one's
+          *reinterpret_cast<uint2*>(&smem[buf][dst_off[i]]) = uint2{reg[set][i].x, reg[set][i].y};
+          *reinterpret_cast<uint2*>(&smem[buf][dst_off[i] + VP]) = uint2{reg[set][i].z, reg[set][i].w};
+        }
+      }
   };
 
   int buf = 0;
 #pragma unroll
-  for (int s2 = 0; s2 < PF; ++s2)
-    if (kb_first + 32 * s2 <= k_hi) load_step(s2);
-  // unrolled by PF so that the register sets are named at compile time: step kb0 + 32 s2 is in set s2
+  for (int s2 = 0; s2 < PF; ++s2) load_step(s2);
+  // whole rounds of PF steps, so that the register sets are named at compile time: step kb0 + 32 s2 is in set
+  // s2; a step past the last key changes nothing (all of it is masked)
   for (int kb0 = kb_first; kb0 <= k_hi; kb0 += 32 * PF) {
 #pragma unroll
     for (int s2 = 0; s2 < PF; ++s2) {
       const int kb = kb0 + 32 * s2;
-      if (kb <= k_hi) {
-        store_step(s2, buf);
-        __syncthreads();
-        if (kb + 32 * PF <= k_hi) load_step(s2);
-        if (head_ok) {
-          const bf16_t* sK = smem[buf];
-          const bf16_t* sV = smem[buf] + SK;
-          f32x4 st[CT][2];
+      store_step(s2, buf);
+      __syncthreads();
+      load_step(s2);
+      if (head_ok) {
+        const bf16_t* sK = smem[buf];
+        const bf16_t* sV = smem[buf] + SK;
+        f32x4 st[CT][2];
 #pragma unroll
-          for (int tt = 0; tt < 2; ++tt) {
+        for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+          for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < KC; ++c) {
-              const uint4 kvv = *reinterpret_cast<const uint4*>(&sK[(tt * 16 + c16) * KP + c * 32 + g * 8]);
-              const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
+          for (int c = 0; c < KC; ++c) {
+            const uint4 kvv = *reinterpret_cast<const uint4*>(&sK[tt * KT + c16 * KP + c * 32 + g * 8]);
+            const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
 #pragma unroll
-              for (int ct = 0; ct < CT; ++ct)
-                st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
-            }
-          }
-          uint4 vraw[DT];
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const uint2 t0 = *reinterpret_cast<const uint2*>(&sV[(0 * DH + dt * 16 + c16) * 16 + 4 * g]);
-            const uint2 t1 = *reinterpret_cast<const uint2*>(&sV[(1 * DH + dt * 16 + c16) * 16 + 4 * g]);
-            vraw[dt] = uint4{t0.x, t0.y, t1.x, t1.y};
-          }
-          if (kb >= all_lo && kb + 31 <= all_hi) {  // the same for the whole wavefront
-            softmax_and_values<DH, CT, false>(st, true, true, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
-          } else {
-            const bool act0 = kb <= k_hi && kb + 15 >= k_lo, act1 = kb + 16 <= k_hi && kb + 31 >= k_lo;
-            softmax_and_values<DH, CT, true>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+            for (int ct = 0; ct < CT; ++ct)
+              st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
           }
         }
-        buf ^= 1;
+        uint4 vraw[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const uint2 t0 = *reinterpret_cast<const uint2*>(&sV[g * VP + (dt * 16 + c16) * 4]);
+          const uint2 t1 = *reinterpret_cast<const uint2*>(&sV[VT + g * VP + (dt * 16 + c16) * 4]);
+          vraw[dt] = uint4{t0.x, t0.y, t1.x, t1.y};
+        }
+        if (kb >= all_lo && kb + 31 <= all_hi) {  // the same for the whole wavefront
+          softmax_and_values<DH, CT, false>(st, true, true, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+        } else {
+          const bool act0 = kb <= k_hi && kb + 15 >= k_lo, act1 = kb + 16 <= k_hi && kb + 31 >= k_lo;
+          softmax_and_values<DH, CT, true>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+        }
       }
+      buf ^= 1;
     }
   }
   if (!head_ok) return;
