@@ -74,12 +74,12 @@ __device__ __forceinline__ void stream_block(const bf16_t* __restrict__ X, const
     xsrc[i] = (uint32_t)(a_rows != nullptr ? a_rows[t] : t) * (uint32_t)K + kc * 8;
     // B operand order: [tile][k step][g][row], the row swizzled by (g, k step)
     const int nt = row >> 4, rr = row & 15, ks = kc >> 2, gg = kc & 3;
-    xdst[i] = (((nt * 2 + ks) * 4 + gg) * 16 + (rr ^ (4 * gg + 2 * ks))) * 8;
+    xdst[i] = (((nt * 2 + ks) * 4 + gg) * 16 + (rr ^ (gg + 4 * ks))) * 8;
   }
   // what this lane reads as B operand: tile nt, k step ks at b_off[ks] + nt * 1024 elements
   int b_off[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) b_off[ks] = ((ks * 4 + g) * 16 + (r ^ (4 * g + 2 * ks))) * 8;
+  for (int ks = 0; ks < 2; ++ks) b_off[ks] = ((ks * 4 + g) * 16 + (r ^ (g + 4 * ks))) * 8;
 
   f32x4 acc0[NTL], acc1[NTL];
 #pragma unroll
