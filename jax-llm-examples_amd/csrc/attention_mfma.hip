@@ -369,16 +369,22 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention
 }
 
 // ------------------------------------------------------------------ prefill portions, heads sharing keys
-// One block per (tile of up to 32 tokens, kv head, up to WAVES of its query heads): a wavefront per
-// query head.  The heads read the same keys and values, so every 32-key step is brought into shared
-// memory once by the whole block (the next step's data is in flight meanwhile) and each wavefront
-// takes its operands from there (laid out so that no access meets another in a bank, see below).
+// A work item is a (tile of up to 32 tokens, query head) pair, one wavefront's worth; a block takes WAVES
+// items of one kv head that follow each other in (tile, head) order, so it spans a few neighbouring tiles of
+// one segment and always has a wavefront for every SIMD (with 5 query heads per kv head, a block per tile
+// would leave one SIMD with twice the work of the others).  The wavefronts read the same keys and values,
+// so every 32-key step of the block's range is brought into shared memory once by the whole block (the
+// next steps' data is in flight meanwhile) and each wavefront takes its operands from there (laid out so
+// that no access meets another in a bank, see below); a wavefront sits out the steps that lie wholly
+// outside its own tile's range.
+//   groups: [num_groups][4] = (first tile, first head within the kv head's group of that tile, items, 0),
+//   longest first; grid = num_groups * Hkv.
 template <int DH, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
+__global__ __launch_bounds__(WAVES * 64, DH <= 128 ? 2 : 1) void attention_prefill_shared_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv, bf16_t* __restrict__ out,
     const int* __restrict__ positions, const int* __restrict__ token_segment, const int* __restrict__ block_table,
-    int table_width, const int* __restrict__ tiles, int num_tiles, int ret_mode, int ret_param, float scale_log2,
-    int Hq, int Hkv, int ps) {
+    int table_width, const int* __restrict__ tiles, const int* __restrict__ groups, int ret_mode, int ret_param,
+    float scale_log2, int Hq, int Hkv, int ps) {
   constexpr int CT = 2, KC = DH / 32, DT = DH / 16;
   constexpr int KP = DH + 8;
   constexpr int THREADS = WAVES * 64;
@@ -395,17 +401,24 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int c16 = lane & 15, g = lane >> 4;
   const int G = Hq / Hkv;
-  const int hchunks = (G + WAVES - 1) / WAVES;
-  const int hc = blockIdx.x % hchunks;
-  const int hk = (blockIdx.x / hchunks) % Hkv;
-  const int tile = num_tiles - 1 - blockIdx.x / (hchunks * Hkv);  // the tiles with the most keys first
-  const int gi = hc * WAVES + wave;
-  const bool head_ok = gi < G;
-  const int h = hk * G + (head_ok ? gi : 0);
+  const int hk = blockIdx.x % Hkv;
+  const int* grp = groups + 4 * (blockIdx.x / Hkv);
+  const int tile0 = grp[0], head0 = grp[1], count = grp[2];
+  // this wavefront's item
+  const bool head_ok = wave < count;
+  const int item = head0 + (head_ok ? wave : 0);
+  const int tile = tile0 + item / G;
+  const int h = hk * G + item % G;
   const int n0 = tiles[2 * tile], nt = tiles[2 * tile + 1];
   const int p_first = positions[n0], p_last = p_first + nt - 1;
-  const int k_lo = first_key(ret_mode, ret_param, p_first);
-  const int k_hi = p_last;
+  const int my_lo = first_key(ret_mode, ret_param, p_first), my_hi = p_last;  // keys any of its tokens may see
+  // the block's range: that of all its tiles
+  int k_lo = INT_MAX, k_hi = 0;
+  for (int t = tile0; t <= tile0 + (head0 + count - 1) / G; ++t) {
+    const int pf = positions[tiles[2 * t]];
+    k_lo = min(k_lo, first_key(ret_mode, ret_param, pf));
+    k_hi = max(k_hi, pf + tiles[2 * t + 1] - 1);
+  }
   const int* table = block_table + (size_t)token_segment[n0] * table_width;
   const size_t plane = (size_t)ps * DH;
   const size_t page_stride = 2 * (size_t)Hkv * plane;
@@ -542,7 +555,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_shared_kernel(
       store_step(s2, buf);
       __syncthreads();
       load_step(s2);
-      if (head_ok) {
+      if (head_ok && kb + 31 >= my_lo && kb <= my_hi) {
         const bf16_t* sK = smem[buf];
         const bf16_t* sV = smem[buf] + SK;
         f32x4 st[CT][2];
@@ -714,14 +727,22 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, c
 
 static bool head_dim_ok(int dh) { return dh == 32 || dh == 64 || dh == 96 || dh == 128 || dh == 256; }
 
+// Wavefronts, and so (tile, head) items, per block of the key-sharing prefill kernel: one per SIMD, and two
+// such blocks fit a compute unit.
+constexpr int kGroupWaves = 4;
+JLE_API int jle_attention_group_waves() { return kGroupWaves; }
+
 JLE_API int jle_attention_mfma_supported(int dh, int Hq, int Hkv, int ps) {
   return head_dim_ok(dh) && Hkv > 0 && Hq % Hkv == 0 && ps >= 16 && ps % 16 == 0;
 }
 
+// groups / num_groups: the packing of (tile, head) items into blocks of kGroupWaves for the kernel that shares
+// keys between the wavefronts of a block (see there; tiles of 32 tokens, more than one query head per kv
+// head); null: one wavefront per item, on its own.
 JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, const int* positions,
                                   const int* token_segment, const int* block_table, int table_width, const int* tiles,
-                                  int num_tiles, int tile_tokens, int ret_mode, int ret_param, float scale, int Hq,
-                                  int Hkv, int dh, int ps, hipStream_t s) {
+                                  int num_tiles, int tile_tokens, const int* groups, int num_groups, int ret_mode,
+                                  int ret_param, float scale, int Hq, int Hkv, int dh, int ps, hipStream_t s) {
   if (num_tiles <= 0) return 0;
   if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps)) return JLE_BAD_ARG;
   if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
@@ -729,22 +750,14 @@ JLE_API int jle_attention_prefill(const void* q, const void* kv, void* out, cons
   dim3 g((unsigned)((items + 3) / 4)), b(256);
   const float sl = scale * kLog2e;
   if (tile_tokens != 16 && tile_tokens != 32) return JLE_BAD_ARG;
-  const int G = Hq / Hkv;
-  if (G >= 2 && tile_tokens == 32) {
-    const int waves = G <= 2 ? 2 : G <= 4 ? 4 : G == 5 ? 5 : 8;
-    const int hchunks = (G + waves - 1) / waves;
-    dim3 gs((unsigned)((long long)num_tiles * Hkv * hchunks));
+  if (groups != nullptr) {
+    if (tile_tokens != 32 || num_groups <= 0) return JLE_BAD_ARG;
+    dim3 gs((unsigned)((long long)num_groups * Hkv));
 #define LAUNCH_S(DH, WV)                                                                                          \
   hipLaunchKernelGGL((attention_prefill_shared_kernel<DH, WV>), gs, dim3(WV * 64), 0, s, (const bf16_t*)q,        \
                      (const bf16_t*)kv, (bf16_t*)out, positions, token_segment, block_table, table_width, tiles,  \
-                     num_tiles, ret_mode, ret_param, sl, Hq, Hkv, ps)
-#define PICK_S(DH)                    \
-  do {                                \
-    if (waves == 2) LAUNCH_S(DH, 2);  \
-    else if (waves == 4) LAUNCH_S(DH, 4); \
-    else if (waves == 5) LAUNCH_S(DH, 5); \
-    else LAUNCH_S(DH, 8);             \
-  } while (0)
+                     groups, ret_mode, ret_param, sl, Hq, Hkv, ps)
+#define PICK_S(DH) LAUNCH_S(DH, kGroupWaves)
     switch (dh) {
       case 32: PICK_S(32); break;
       case 64: PICK_S(64); break;

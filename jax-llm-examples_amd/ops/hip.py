@@ -31,7 +31,7 @@ _SIGNATURES = {
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
-    "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
+    "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
     "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i,
                              _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -72,6 +72,7 @@ def load_library():
             fn.restype = ctypes.c_int
         lib.jle_attention_mfma_supported.argtypes = [_i, _i, _i, _i]  # a query, not a launch: no stream
         lib.jle_gemm_stream_supported.argtypes = [_i, _i, _i]
+        lib.jle_attention_group_waves.argtypes = []
         lib._jle_path = path
         _LIB = lib
     return _LIB
@@ -321,21 +322,24 @@ class HipOps:
     DECODE_FIT_SPLIT = 1024  # ... at most, to make the items fit in one go
     DECODE_MAX_SPLIT = 512  # ... when there are more items than fit anyway
 
-    def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1):
+    def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1, group_size=1):
         """Work lists of the MFMA attention kernels for one step and one retention rule: the rows that are
-        single decode tokens (and into how many keys their work is split), and tiles of up to 32
-        consecutive tokens of longer segments."""
+        single decode tokens (and into how many keys their work is split), tiles of up to 32 consecutive
+        tokens of longer segments and, with ``group_size`` > 1 query heads per kv head, the packing of the
+        (tile, head) items of a kv head into blocks of wavefronts that share keys."""
         from ..parts.base import first_needed_position
 
-        dec, tiles, spans = [], [], []
+        dec, tiles, spans, seg_tiles = [], [], [], []
         o = 0
         for n, start in zip(seg_lens, seg_starts):
             if n == 1:
                 dec.append(o)
                 spans.append((first_needed_position(retention, start), start))
             else:
+                first = len(tiles) // 2
                 for t in range(0, n, self.PREFILL_TILE):
                     tiles += [o + t, min(self.PREFILL_TILE, n - t)]
+                seg_tiles.append((first, len(tiles) // 2 - first, start + n - 1))
             o += n
         split, max_splits = self.DECODE_MAX_SPLIT, 1
         if dec:
@@ -346,9 +350,26 @@ class HipOps:
                     split = cand
                     break
             max_splits = max(p // split - f // split + 1 for f, p in spans)
-        flat = torch.tensor(dec + tiles, dtype=torch.int32).to(device) if dec or tiles else None
-        return {"num_dec": len(dec), "num_tiles": len(tiles) // 2, "max_splits": max_splits, "split": split,
-                "dec": flat[: len(dec)] if dec else None, "tiles": flat[len(dec):] if tiles else None}
+        groups = []
+        if tiles and group_size > 1 and self.PREFILL_TILE == 32:
+            # consecutive (tile, head) items of one segment, `waves` per block; blocks with the most keys first
+            waves = int(self.lib.jle_attention_group_waves())
+            keyed = []
+            for first, count, last_pos in seg_tiles:
+                items = count * group_size
+                for lo in range(0, items, waves):
+                    n_items = min(waves, items - lo)
+                    last_tile = first + (lo + n_items - 1) // group_size
+                    end = last_pos - (first + count - 1 - last_tile) * self.PREFILL_TILE  # about where its keys end
+                    keyed.append((-end, len(keyed), [first + lo // group_size, lo % group_size, n_items, 0]))
+            keyed.sort()
+            groups = [v for _, _, quad in keyed for v in quad]
+        flat = dec + tiles + groups
+        flat = torch.tensor(flat, dtype=torch.int32).to(device) if flat else None
+        nd, nt = len(dec), len(tiles)
+        return {"num_dec": nd, "num_tiles": nt // 2, "max_splits": max_splits, "split": split,
+                "dec": flat[:nd] if dec else None, "tiles": flat[nd: nd + nt] if tiles else None,
+                "groups": flat[nd + nt:] if groups else None, "num_groups": len(groups) // 4}
 
     def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
         n, hq, dh = q.shape
@@ -363,7 +384,8 @@ class HipOps:
         out = torch.empty(n, hq * dh, dtype=q.dtype, device=q.device)
         if (q.dtype == torch.bfloat16 and hq // hk <= 32
                 and self.lib.jle_attention_mfma_supported(dh, hq, hk, ps)):
-            plan = meta.meta.get("attn_plan") if meta is not None else None
+            key = f"attn_plan_{hq // hk}"
+            plan = meta.meta.get(key) if meta is not None else None
             if plan is None:
                 if meta is not None:
                     seg_lens, seg_starts = meta.seg_lens, meta.seg_starts
@@ -376,13 +398,14 @@ class HipOps:
                             seg_lens.append(0)
                             seg_starts.append(pos[i])
                         seg_lens[-1] += 1
-                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk)
+                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk, hq // hk)
                 if meta is not None:
-                    meta.meta["attn_plan"] = plan
+                    meta.meta[key] = plan
             if plan["num_tiles"]:
                 self._call("jle_attention_prefill", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
                            _p(block_table), block_table.shape[1], _p(plan["tiles"]), plan["num_tiles"],
-                           self.PREFILL_TILE, mode, param, float(scale), hq, hk, dh, ps)
+                           self.PREFILL_TILE, _p(plan["groups"]), plan["num_groups"], mode, param, float(scale), hq,
+                           hk, dh, ps)
             if plan["num_dec"]:
                 cols = 16 if hq // hk <= 16 else 32
                 items = plan["num_dec"] * hk * plan["max_splits"]
