@@ -177,7 +177,7 @@ __device__ __forceinline__ void stream_block(const bf16_t* __restrict__ X, const
 }
 
 template <bool SWIGLU, typename OutT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void gemm_stream_kernel(const bf16_t* __restrict__ X,
+__global__ __launch_bounds__(WAVES * 64, 2) void gemm_stream_kernel(const bf16_t* __restrict__ X,
                                                                  const bf16_t* __restrict__ W, OutT* __restrict__ Y,
                                                                  const int* __restrict__ offsets,
                                                                  const int* __restrict__ a_rows,
@@ -241,47 +241,27 @@ JLE_API int jle_gemm_stream_supported(int Nout, int K, int swiglu) {
 }
 
 // X [*, K] bf16, W [G, Nout, K] bf16 in the streaming layout, Y [M, Nout] (or [M, Nout / 2] with swiglu) bf16 or
-// float32; X must have fewer than 2^32 elements.  max_rows: the most rows any group can have (M if unknown).  waves: wavefronts per block (4, 5, 6 or
-// 8; 0 = chosen from the sizes so that the blocks come out in whole rounds over the compute units).
+// float32; X must have fewer than 2^32 elements.  max_rows: the most rows any group can have (M if unknown).
+// Blocks are 8 wavefronts (two per SIMD, one block per compute unit): measured against 4, 5 and 6 on expert
+// shapes with even and with skewed numbers of rows per expert.
 JLE_API int jle_gemm_stream(const void* X, const void* W, void* Y, const int* offsets, const int* a_rows,
                             const float* scale, int swiglu, int out_f32, int M, int Nout, int K, int G, int max_rows,
-                            int waves, hipStream_t s) {
+                            hipStream_t s) {
   if (M <= 0 || Nout <= 0) return 0;
   if (G < 1 || G > 65535 || !jle_gemm_stream_supported(Nout, K, swiglu)) return JLE_BAD_ARG;
   if (max_rows <= 0 || max_rows > M) max_rows = M;
+  constexpr int kWaves = 8;
   const int passes = (max_rows + kRows - 1) / kRows;
   const int pairs = swiglu ? Nout / 32 : (Nout / 16 + 1) / 2;  // pairs of weight tiles = wavefronts needed per group
-  if (waves == 0) {
-    // one block per compute unit at a time: prefer the size whose last round is fullest
-    const long long groups = offsets != nullptr ? (G < M ? G : M) : 1;
-    double best = -1.0;
-    const int cand[4] = {8, 6, 5, 4};
-    for (int c = 0; c < 4; ++c) {
-      const long long blocks = (long long)((pairs + cand[c] - 1) / cand[c]) * groups;
-      const long long rounds = (blocks + 255) / 256;
-      const double fill = (double)blocks / (double)(rounds * 256) * (cand[c] >= 6 ? 1.0 : 0.9);
-      if (fill > best + 1e-9) {
-        best = fill;
-        waves = cand[c];
-      }
-    }
-  }
-  if (waves != 4 && waves != 5 && waves != 6 && waves != 8) return JLE_BAD_ARG;
-  const int nblk = (pairs + waves - 1) / waves;
+  const int nblk = (pairs + kWaves - 1) / kWaves;
   if ((long long)nblk * passes * G > (1ll << 30)) return JLE_BAD_ARG;
-#define PICK(SW, OT)                                                                              \
-  do {                                                                                            \
-    if (waves == 8) launch_stream<SW, OT, 8>(nblk, passes, G, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);      \
-    else if (waves == 6) launch_stream<SW, OT, 6>(nblk, passes, G, s, X, W, Y, offsets, a_rows, scale, M, Nout, K); \
-    else if (waves == 5) launch_stream<SW, OT, 5>(nblk, passes, G, s, X, W, Y, offsets, a_rows, scale, M, Nout, K); \
-    else launch_stream<SW, OT, 4>(nblk, passes, G, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);                 \
-  } while (0)
   if (swiglu) {
-    if (out_f32) PICK(true, float); else PICK(true, bf16_t);
+    if (out_f32) launch_stream<true, float, kWaves>(nblk, passes, G, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);
+    else launch_stream<true, bf16_t, kWaves>(nblk, passes, G, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);
   } else {
-    if (out_f32) PICK(false, float); else PICK(false, bf16_t);
+    if (out_f32) launch_stream<false, float, kWaves>(nblk, passes, G, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);
+    else launch_stream<false, bf16_t, kWaves>(nblk, passes, G, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);
   }
-#undef PICK
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -36,7 +36,7 @@ _SIGNATURES = {
                              _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
-    "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
 
@@ -252,8 +252,7 @@ class HipOps:
     def stream_supported(self, nout: int, k: int, swiglu: bool) -> bool:
         return bool(self.lib.jle_gemm_stream_supported(nout, k, int(swiglu)))
 
-    def gemm_stream(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
-                    waves: int = 0):
+    def gemm_stream(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None):
         """bfloat16 product on MFMA for about a hundred rows per group, weights in the streaming layout and
         read once per 192 rows of a group (see ``gemm_stream.hip``)."""
         if b.dim() == 2:
@@ -272,7 +271,7 @@ class HipOps:
         out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
                           device=a.device)
         self._call("jle_gemm_stream", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
-                   int(out_f32), m, nout, k, g, m, int(waves))
+                   int(out_f32), m, nout, k, g, m)
         return out
 
     def lm_head(self, h, w, tiled: bool = False):

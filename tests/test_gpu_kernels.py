@@ -432,11 +432,10 @@ def test_grouped_product_for_many_rows(ops, ref, n, d, f, e, k):
     assert head.dtype == torch.float32 and head.shape == (100, 311)
 
 
-@pytest.mark.parametrize("n,d,f,e,k,waves", [(300, 256, 32, 16, 1, 0), (700, 768, 96, 3, 2, 5), (2048, 512, 256, 16, 1, 8),
-                                             (150, 256, 48, 128, 1, 4), (900, 256, 80, 2, 1, 6)])
-def test_weight_streaming_grouped_product(ops, ref, n, d, f, e, k, waves):
-    """Groups without rows, with a few, with more than one pass of 256; an odd number of weight tiles; every
-    block size."""
+@pytest.mark.parametrize("n,d,f,e,k", [(300, 256, 32, 16, 1), (700, 768, 96, 3, 2), (2048, 512, 256, 16, 1),
+                                       (150, 256, 48, 128, 1), (900, 256, 80, 2, 1)])
+def test_weight_streaming_grouped_product(ops, ref, n, d, f, e, k):
+    """Groups without rows, with a few, with more than one pass of 192; an odd number of weight tiles."""
     from jax_llm_examples_amd.ops.layout import tile_
     dt = torch.bfloat16
     h = _rand(n, d, dt=dt, seed=1)
@@ -451,24 +450,24 @@ def test_weight_streaming_grouped_product(ops, ref, n, d, f, e, k, waves):
     wgu_t = wgu.clone()
     tile_(wgu_t)
     gu = ops.gemm(h, wgu, offsets=off, a_rows=tok, scale=gate, out_f32=True)  # the general kernel, float32 result
-    plain = ops.gemm_stream(h, wgu_t, offsets=off, a_rows=tok, scale=gate, out_f32=True, waves=waves)
+    plain = ops.gemm_stream(h, wgu_t, offsets=off, a_rows=tok, scale=gate, out_f32=True)
     assert float((plain - gu).abs().max() / gu.abs().max()) <= 2e-5
     if f % 16 == 0:
-        act = ops.gemm_stream(h, wgu_t, offsets=off, a_rows=tok, scale=gate, swiglu=True, waves=waves)
+        act = ops.gemm_stream(h, wgu_t, offsets=off, a_rows=tok, scale=gate, swiglu=True)
         want = torch.nn.functional.silu(gu[:, :f]) * gu[:, f:]
         assert act.shape == (n * k, f)
         assert float((act.float() - want).abs().max() / want.abs().max()) <= 5e-3
     else:
         with pytest.raises(Exception, match="refuses|needs"):
-            ops.gemm_stream(h, wgu_t, offsets=off, a_rows=tok, scale=gate, swiglu=True, waves=waves)
+            ops.gemm_stream(h, wgu_t, offsets=off, a_rows=tok, scale=gate, swiglu=True)
         act = ops.gemm_grouped(h, wgu, offsets=off, a_rows=tok, scale=gate, swiglu=True)
     if f % 256 == 0:
         wd_t = wd.clone()
         tile_(wd_t)
-        down = ops.gemm_stream(act, wd_t, offsets=off, waves=waves)
+        down = ops.gemm_stream(act, wd_t, offsets=off)
         want_d = ops.gemm(act, wd, offsets=off, out_f32=True)
         assert float((down.float() - want_d).abs().max() / want_d.abs().max()) <= 5e-3
-    dense = ops.gemm_stream(h, wgu_t[0], out_f32=True, waves=waves)  # one group, no offsets
+    dense = ops.gemm_stream(h, wgu_t[0], out_f32=True)  # one group, no offsets
     assert float((dense - h.float() @ wgu[0].float().t()).abs().max() / dense.abs().max()) <= 2e-5
     with pytest.raises(Exception, match="refuses|needs"):
         ops.gemm_stream(h[:, :d - 128].contiguous(), wgu_t[:, :, :d - 128].contiguous())
