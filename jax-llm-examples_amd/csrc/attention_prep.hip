@@ -79,12 +79,155 @@ __global__ void qk_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
   }
 }
 
+// The same for head sizes of 16, 32, 64, 128, 256 or 512 (all sizes a power of two), with 16- or 32-byte
+// accesses: a lane takes 8 consecutive elements (4 pairs) of a head, head_dim / 8 lanes a head, so a wavefront
+// takes 64 / (head_dim / 8) heads at a time and goes through up to kRounds such sets of consecutive heads of
+// one token: the sines and cosines of the lane's pairs are the token's, formed once.
+constexpr int kRounds = 4;
+
+template <typename T>
+struct Vec8;
+template <>
+struct Vec8<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const uint4 r = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+    *reinterpret_cast<uint4*>(p) =
+        uint4{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+  }
+};
+template <>
+struct Vec8<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
+    *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<float4*>(p + 4) = float4{v[4], v[5], v[6], v[7]};
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_prepare_vec_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
+                                                             T* __restrict__ kv_cache,
+                                                             const int* __restrict__ positions,
+                                                             const int* __restrict__ slot_mapping,
+                                                             const float* __restrict__ inv_freq, float norm_eps,
+                                                             float floor_scale, float attn_scale, int N, int Hq,
+                                                             int Hkv, int dh, int page_size, int write_kv) {
+  const int lane = threadIdx.x & 63;
+  const int H = Hq + 2 * Hkv;
+  const int H_here = write_kv ? H : Hq;
+  const int lph = dh >> 3;          // lanes per head
+  const int hps = 64 / lph;         // heads per set
+  const int per_wave = hps * kRounds;
+  const int per_token = (H_here + per_wave - 1) / per_wave;  // wavefronts per token; four wavefronts a block
+  const int item = blockIdx.x * 4 + wave_index();
+  const int n = item / per_token;
+  if (n >= N) return;
+  const int h_base = (item - n * per_token) * per_wave;
+  const int sub = lane / lph, l = lane - sub * lph;  // head of the set, place within the head
+  const int pos = positions[n];
+  float sn[4], cs[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    sn[i] = 0.f;
+    cs[i] = 1.f;
+    if (inv_freq != nullptr) {
+      const float ang = (float)pos * inv_freq[4 * l + i];
+      sn[i] = sinf(ang);
+      cs[i] = cosf(ang);
+    }
+  }
+  float q_mul = 1.f;
+  if (floor_scale > 0.f) q_mul = 1.0f + attn_scale * log1pf(floorf(((float)pos + 1.0f) / floor_scale));
+  int page = 0, off = 0;
+  if (write_kv) {
+    const int slot = slot_mapping[n];
+    page = slot / page_size;
+    off = slot - page * page_size;
+  }
+  float x[kRounds][8];
+  bool live[kRounds];
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {  // everything is asked for before the first head is worked on
+    const int h = h_base + r * hps + sub;
+    live[r] = h < H_here;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[r][i] = 0.f;
+    if (live[r]) Vec8<T>::load(qkv + ((size_t)n * H + h) * dh + 8 * l, x[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const int h = h_base + r * hps + sub;
+    const bool is_q = h < Hq, is_v = h >= Hq + Hkv;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float x1 = x[r][2 * i], x2 = x[r][2 * i + 1];
+      if (!is_v && inv_freq != nullptr) {
+        const float r1 = x1 * cs[i] - x2 * sn[i];
+        const float r2 = x2 * cs[i] + x1 * sn[i];
+        x1 = r1;
+        x2 = r2;
+      }
+      x[r][2 * i] = x1;
+      x[r][2 * i + 1] = x2;
+      ss += x1 * x1 + x2 * x2;
+    }
+    float mul = 1.f;
+    if (norm_eps >= 0.f) {  // over the head's lanes (all lanes take part; a value head ignores the result)
+      for (int o = lph >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      if (!is_v) mul = 1.0f / sqrtf(ss / (float)dh + norm_eps);
+    }
+    if (is_q) mul *= q_mul;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[r][i] *= mul;
+    if (!live[r]) continue;
+    if (is_v) {  // one element of all the page's tokens is contiguous: this token's elements are page_size apart
+      T* dst = kv_cache + (((size_t)page * 2 + 1) * Hkv + (h - Hq - Hkv)) * page_size * dh + off;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) Num<T>::store(dst + (size_t)(8 * l + i) * page_size, x[r][i]);
+    } else {
+      T* dst = is_q ? q_out + ((size_t)n * Hq + h) * dh
+                    : kv_cache + (((size_t)page * 2) * Hkv + (h - Hq)) * page_size * dh + (size_t)off * dh;
+      Vec8<T>::store(dst + 8 * l, x[r]);
+    }
+  }
+}
+
 JLE_API int jle_qk_prepare(const void* qkv, void* q_out, void* kv_cache, const int* positions,
                            const int* slot_mapping, const float* inv_freq, float norm_eps, float floor_scale,
                            float attn_scale, int is_bf16, int N, int Hq, int Hkv, int dh, int page_size,
                            int write_kv, hipStream_t s) {
   if (N <= 0) return 0;
   if (dh % 2 || dh > 128 * kMaxPairsPerLane || Hq + 2 * Hkv > 65535) return JLE_BAD_ARG;
+  const bool aligned = (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)kv_cache) & 31) == 0;
+  if (aligned && dh >= 16 && dh <= 512 && (dh & (dh - 1)) == 0) {  // whatever N: a token's result is the same
+    const int per_wave = (64 / (dh / 8)) * kRounds;
+    const int H_here = write_kv ? Hq + 2 * Hkv : Hq;
+    const long long waves = (long long)N * ((H_here + per_wave - 1) / per_wave);
+    if (waves > (1ll << 31)) return JLE_BAD_ARG;
+    dim3 gv((unsigned)((waves + 3) / 4)), bv(256);
+    if (is_bf16)
+      hipLaunchKernelGGL(qk_prepare_vec_kernel<bf16_t>, gv, bv, 0, s, (const bf16_t*)qkv, (bf16_t*)q_out,
+                         (bf16_t*)kv_cache, positions, slot_mapping, inv_freq, norm_eps, floor_scale, attn_scale, N,
+                         Hq, Hkv, dh, page_size, write_kv);
+    else
+      hipLaunchKernelGGL(qk_prepare_vec_kernel<float>, gv, bv, 0, s, (const float*)qkv, (float*)q_out,
+                         (float*)kv_cache, positions, slot_mapping, inv_freq, norm_eps, floor_scale, attn_scale, N, Hq,
+                         Hkv, dh, page_size, write_kv);
+    JLE_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 g(N, Hq + 2 * Hkv), b(64);
   if (is_bf16)
     hipLaunchKernelGGL(qk_prepare_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)kv_cache,

@@ -84,6 +84,25 @@ def test_silu_mul_gather_add(ops, ref, dt):
     assert torch.allclose(r, want, rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("dt", DT)
+def test_qk_prepare_of_a_token_does_not_depend_on_the_batch(ops, ref, dt):
+    """Many tokens take wavefronts that go through several heads each; the results must be those of a token
+    prepared alone, bit for bit."""
+    hq, hk, dh, n, ps = 40, 8, 128, 320, 16
+    qkv, pos, pages, slots, inv_freq = _prep_case(hq, hk, dh, n, ps, dt)
+    c1 = torch.zeros(pages, 2, hk, ps, dh, dtype=dt, device=DEV)
+    c2, c3 = c1.clone(), c1.clone()
+    q1 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq, 1e-5, (16.0, 0.1), c1, slots)
+    q2 = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq, 1e-5, (16.0, 0.1), c2, slots)
+    assert torch.allclose(q1.float(), q2.float(), **_tol(dt)) and torch.allclose(c1.float(), c2.float(), **_tol(dt))
+    few = slice(100, 107)
+    q3 = ops.qk_prepare_kv_write(qkv[few].contiguous(), hq, hk, dh, pos[few].contiguous(), inv_freq, 1e-5,
+                                 (16.0, 0.1), c3, slots[few].contiguous())
+    assert torch.equal(q3, q1[few])
+    written = c3 != 0
+    assert written.any() and torch.equal(c3[written], c1[written])
+
+
 def _prep_case(hq, hk, dh, n, ps, dt, seed=0):
     qkv = _rand(n, (hq + 2 * hk) * dh, dt=dt, seed=seed)
     pos = torch.randint(0, 500, (n,), generator=torch.Generator().manual_seed(seed)).to(torch.int32).to(DEV)
