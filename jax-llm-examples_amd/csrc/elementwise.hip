@@ -3,6 +3,8 @@
 
 using namespace jle;
 
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
 // ------------------------------------------------------------------ embedding
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ tok, const T* __restrict__ table, float* __restrict__ out, int D) {
@@ -85,6 +87,84 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_reg_kernel(float* __restr
   }
 }
 
+// four neighbouring elements
+template <typename T>
+__device__ __forceinline__ f32x4_t load4(const T* p);
+template <>
+__device__ __forceinline__ f32x4_t load4<float>(const float* p) {
+  return *reinterpret_cast<const f32x4_t*>(p);
+}
+template <>
+__device__ __forceinline__ f32x4_t load4<bf16_t>(const bf16_t* p) {
+  const uint2 r = *reinterpret_cast<const uint2*>(p);
+  return f32x4_t{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
+                 __uint_as_float(r.y & 0xffff0000u)};
+}
+template <typename T>
+__device__ __forceinline__ void store4(T* p, f32x4_t v);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, f32x4_t v) {
+  *reinterpret_cast<f32x4_t*>(p) = v;
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v) {
+  *reinterpret_cast<uint2*>(p) = uint2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+}
+
+template <typename DT>
+__device__ __forceinline__ f32x4_t delta_at4(const Delta<DT>& delta, size_t n, int d, int D) {
+  f32x4_t v = {0.f, 0.f, 0.f, 0.f};
+  if (delta.plain != nullptr) v = load4<DT>(delta.plain + n * D + d);
+  if (delta.routed != nullptr) {
+    for (int j = 0; j < delta.k; ++j) v += load4<DT>(delta.routed + (size_t)delta.inv[n * delta.k + j] * D + d);
+    if (delta.shared != nullptr) v += load4<DT>(delta.shared + n * D + d);
+  }
+  return v;
+}
+
+// Rows whose width is a multiple of 8 (and 16-byte aligned arrays): a thread takes CPT pieces of 4
+// neighbouring elements, piece = thread, thread + THREADS, ...; up to THREADS * CPT * 4 wide.
+template <typename DT, typename OT, int THREADS, int CPT>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ x, Delta<DT> delta,
+                                                                  const float* __restrict__ w, float eps,
+                                                                  OT* __restrict__ out, float* __restrict__ out32,
+                                                                  int D) {
+  __shared__ float red[THREADS / 64];
+  const size_t n = blockIdx.x;
+  const size_t base = n * D;
+  f32x4_t v[CPT];
+  float ss = 0.f;
+  const bool add = delta.any();
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int d = (threadIdx.x + THREADS * i) * 4;
+    v[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (d < D) {
+      v[i] = load4<float>(x + base + d);
+      if (add) {
+        v[i] += delta_at4<DT>(delta, n, d, D);
+        store4<float>(x + base + d, v[i]);
+      }
+      ss += v[i][0] * v[i][0];
+      ss += v[i][1] * v[i][1];
+      ss += v[i][2] * v[i][2];
+      ss += v[i][3] * v[i][3];
+    }
+  }
+  const float tot = block_sum<THREADS>(ss, red);
+  const float inv = 1.0f / sqrtf(tot / (float)D + eps);
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int d = (threadIdx.x + THREADS * i) * 4;
+    if (d < D) {
+      f32x4_t h = v[i] * inv;
+      if (w != nullptr) h *= load4<float>(w + d);
+      if (out != nullptr) store4<OT>(out + base + d, h);
+      if (out32 != nullptr) store4<float>(out32 + base + d, h);
+    }
+  }
+}
+
 template <typename DT, typename OT>
 __global__ __launch_bounds__(256) void add_rmsnorm_wide_kernel(float* __restrict__ x, Delta<DT> delta,
                                                                const float* __restrict__ w, float eps,
@@ -117,7 +197,13 @@ template <typename DT, typename OT>
 static void launch_add_rmsnorm(float* x, Delta<DT> delta, const float* w, float eps, void* out, float* out32, int N,
                                int D, hipStream_t s) {
   dim3 g(N);
-  if (D <= 1024)
+  // (which kernel: by the width and the arrays' alignment only, so a row's result is the same in any batch)
+  const uintptr_t all = (uintptr_t)x | (uintptr_t)delta.plain | (uintptr_t)delta.routed | (uintptr_t)delta.shared |
+                        (uintptr_t)w | (uintptr_t)out | (uintptr_t)out32;
+  if (D % 8 == 0 && (all & 15) == 0 && D > 1024 && D <= 8192)  // (rows of any of the arrays then start 16-byte aligned)
+    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<DT, OT, 256, 8>), g, dim3(256), 0, s, x, delta, w, eps, (OT*)out, out32,
+                       D);
+  else if (D <= 1024)
     hipLaunchKernelGGL((add_rmsnorm_reg_kernel<DT, OT, 256, 4>), g, dim3(256), 0, s, x, delta, w, eps, (OT*)out, out32,
                        D);
   else if (D <= 8192)

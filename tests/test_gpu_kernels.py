@@ -48,7 +48,7 @@ def test_embed(ops, ref, dt):
 
 
 @pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("d", [80, 1000, 1026, 5120, 9000])
+@pytest.mark.parametrize("d", [80, 1000, 1026, 1028, 2056, 5120, 8192, 9000])
 def test_add_rmsnorm(ops, ref, dt, d):
     for delta_dt, weighted, want32 in [(None, True, False), (dt, True, True), (torch.float32, False, True)]:
         x = _rand(7, d, seed=1)
