@@ -81,9 +81,9 @@ __global__ void qk_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
 
 // The same for head sizes of 16, 32, 64, 128, 256 or 512 (all sizes a power of two), with 16- or 32-byte
 // accesses: a lane takes 8 consecutive elements (4 pairs) of a head, head_dim / 8 lanes a head, so a wavefront
-// takes 64 / (head_dim / 8) heads at a time and goes through up to kRounds such sets of consecutive heads of
-// one token: the sines and cosines of the lane's pairs are the token's, formed once.
-constexpr int kRounds = 4;
+// takes 64 / (head_dim / 8) heads at a time and goes through ROUNDS such sets of consecutive heads of one
+// token: the sines and cosines of the lane's pairs are the token's, formed once (ROUNDS is 4 for many tokens,
+// 1 for few, where more wavefronts matter more; a head's result does not depend on it).
 
 template <typename T>
 struct Vec8;
@@ -115,7 +115,7 @@ struct Vec8<float> {
   }
 };
 
-template <typename T>
+template <typename T, int ROUNDS>
 __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                                              T* __restrict__ kv_cache,
                                                              const int* __restrict__ positions,
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(const T* __restrict
   const int H_here = write_kv ? H : Hq;
   const int lph = dh >> 3;          // lanes per head
   const int hps = 64 / lph;         // heads per set
-  const int per_wave = hps * kRounds;
+  const int per_wave = hps * ROUNDS;
   const int per_token = (H_here + per_wave - 1) / per_wave;  // wavefronts per token; four wavefronts a block
   const int item = blockIdx.x * 4 + wave_index();
   const int n = item / per_token;
@@ -155,10 +155,10 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(const T* __restrict
     page = slot / page_size;
     off = slot - page * page_size;
   }
-  float x[kRounds][8];
-  bool live[kRounds];
+  float x[ROUNDS][8];
+  bool live[ROUNDS];
 #pragma unroll
-  for (int r = 0; r < kRounds; ++r) {  // everything is asked for before the first head is worked on
+  for (int r = 0; r < ROUNDS; ++r) {  // everything is asked for before the first head is worked on
     const int h = h_base + r * hps + sub;
     live[r] = h < H_here;
 #pragma unroll
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(const T* __restrict
     if (live[r]) Vec8<T>::load(qkv + ((size_t)n * H + h) * dh + 8 * l, x[r]);
   }
 #pragma unroll
-  for (int r = 0; r < kRounds; ++r) {
+  for (int r = 0; r < ROUNDS; ++r) {
     const int h = h_base + r * hps + sub;
     const bool is_q = h < Hq, is_v = h >= Hq + Hkv;
     float ss = 0.f;
@@ -212,19 +212,21 @@ JLE_API int jle_qk_prepare(const void* qkv, void* q_out, void* kv_cache, const i
   if (dh % 2 || dh > 128 * kMaxPairsPerLane || Hq + 2 * Hkv > 65535) return JLE_BAD_ARG;
   const bool aligned = (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)kv_cache) & 31) == 0;
   if (aligned && dh >= 16 && dh <= 512 && (dh & (dh - 1)) == 0) {  // whatever N: a token's result is the same
-    const int per_wave = (64 / (dh / 8)) * kRounds;
     const int H_here = write_kv ? Hq + 2 * Hkv : Hq;
+    const int rounds = (long long)N * H_here >= 8192 ? 4 : 1;
+    const int per_wave = (64 / (dh / 8)) * rounds;
     const long long waves = (long long)N * ((H_here + per_wave - 1) / per_wave);
     if (waves > (1ll << 31)) return JLE_BAD_ARG;
     dim3 gv((unsigned)((waves + 3) / 4)), bv(256);
-    if (is_bf16)
-      hipLaunchKernelGGL(qk_prepare_vec_kernel<bf16_t>, gv, bv, 0, s, (const bf16_t*)qkv, (bf16_t*)q_out,
-                         (bf16_t*)kv_cache, positions, slot_mapping, inv_freq, norm_eps, floor_scale, attn_scale, N,
-                         Hq, Hkv, dh, page_size, write_kv);
-    else
-      hipLaunchKernelGGL(qk_prepare_vec_kernel<float>, gv, bv, 0, s, (const float*)qkv, (float*)q_out,
-                         (float*)kv_cache, positions, slot_mapping, inv_freq, norm_eps, floor_scale, attn_scale, N, Hq,
-                         Hkv, dh, page_size, write_kv);
+#define LAUNCH_V(T, R)                                                                                            \
+  hipLaunchKernelGGL((qk_prepare_vec_kernel<T, R>), gv, bv, 0, s, (const T*)qkv, (T*)q_out, (T*)kv_cache, positions, \
+                     slot_mapping, inv_freq, norm_eps, floor_scale, attn_scale, N, Hq, Hkv, dh, page_size, write_kv)
+    if (is_bf16) {
+      if (rounds == 4) LAUNCH_V(bf16_t, 4); else LAUNCH_V(bf16_t, 1);
+    } else {
+      if (rounds == 4) LAUNCH_V(float, 4); else LAUNCH_V(float, 1);
+    }
+#undef LAUNCH_V
     JLE_LAUNCH_CHECK();
     return 0;
   }
