@@ -247,7 +247,6 @@ class HipOps:
                    int(out_f32), m, nout, k, g, int(tiled))
         return out
 
-    STREAM_MAX_ROWS = 160  # rows per group, on average, up to which the weight-streaming grouped product is used
 
     def stream_supported(self, nout: int, k: int, swiglu: bool) -> bool:
         return bool(self.lib.jle_gemm_stream_supported(nout, k, int(swiglu)))
@@ -461,10 +460,9 @@ class HipOps:
             act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,
                                    tiled=tiled)
             routed = self.gemm_skinny(act, w_down, offsets=offsets, tiled=tiled)
-        elif (mfma and tiled and n * k <= self.STREAM_MAX_ROWS * e and self.stream_supported(f2, d, True)
-              and self.stream_supported(d, f2 // 2, False)):
-            # around a hundred rows per expert: still bound by reading the weights, which this kernel reads once
-            # per 192 rows of an expert
+        elif mfma and tiled and self.stream_supported(f2, d, True) and self.stream_supported(d, f2 // 2, False):
+            # around a hundred rows per expert the cost is reading the weights, which this kernel reads once per
+            # 192 rows of an expert; with more rows it is still the faster one (measured up to 1024 per expert)
             act = self.gemm_stream(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True)
             routed = self.gemm_stream(act, w_down, offsets=offsets)
         elif mfma:
