@@ -278,8 +278,13 @@ class HipOps:
         if h.dtype == torch.float32:
             return torch.matmul(h, w.t())
         if h.shape[1] % 8 == 0:
-            if h.shape[0] <= self.SKINNY_MAX_ROWS:
+            streams = tiled and self.stream_supported(w.shape[0], w.shape[1], False)
+            # measured on a 202048 x 5120 head: up to 16 rows the skinny kernel is at the speed of reading the
+            # weights; beyond, the kernel that shares the rows between wavefronts through shared memory
+            if h.shape[0] <= (16 if streams else self.SKINNY_MAX_ROWS):
                 return self.gemm_skinny(h, w, out_f32=True, tiled=tiled)
+            if streams:
+                return self.gemm_stream(h, w, out_f32=True)
             return self.gemm_grouped(h, w, out_f32=True, tiled=tiled)
         return self.gemm(h, w, out_f32=True)
 
