@@ -15,8 +15,9 @@ import traces
 from jax_llm_examples_amd.cache import CacheManager, CacheView
 from jax_llm_examples_amd.config import ModelPlan, OrderEntry, LayerSpec, part, register_architecture
 from jax_llm_examples_amd.engine import ModelRunner, StepEntry, build_context, get_ops, load_model
-from jax_llm_examples_amd.parts import (CacheNeed, DecoderModel, Mixer, ParamSpec, build_feed_forward, build_mixer,
-                                        build_norm, register_mixer)
+from jax_llm_examples_amd.parts import (CacheNeed, DecoderModel, FeedForward, Mixer, ParamSpec, PositionEncoding,
+                                        build_feed_forward, build_mixer, build_norm, build_position,
+                                        register_feed_forward, register_mixer, register_position)
 from jax_llm_examples_amd.parts.residual import Residual
 from jax_llm_examples_amd.weights import TensorBinding, init_random_
 from tiny_configs import tiny_config_json
@@ -243,6 +244,132 @@ def test_toy_mixer_with_state_runs_and_does_not_depend_on_the_cut(device):
     got = model.blocks[0].mixer.forward(h.to(device), Ctx(_ops(device), torch.tensor([0]), [len(toks)]),
                                         CacheView(0, True, state=state))
     assert torch.allclose(got.cpu(), direct, rtol=1e-4, atol=1e-5)
+
+
+# ------------------------------------------------ a toy feed-forward with routing, a toy position encoding
+@register_feed_forward("toy_parity_experts")
+class ToyParityExperts(FeedForward):
+    """Two linear experts; a token goes to the one named by the sign of a fixed direction of its float32 row
+    (routing of its own, nothing of the MoE part), and the output is scaled by a gate from the same number."""
+
+    wants_float32_input = True
+
+    def __init__(self, spec):
+        super().__init__()
+        self.hidden = int(spec.hidden_size)
+
+    def param_specs(self):
+        return {"direction": ParamSpec((self.hidden,), policy="float32"),
+                "experts": ParamSpec((2, self.hidden, self.hidden))}
+
+    def forward(self, h, h32, ctx):
+        score = h32 @ self.params["direction"]
+        which = (score > 0).long()
+        w = self.params["experts"][which].float()  # [N, D, D]
+        out = torch.einsum("nij,nj->ni", w, h.float()) * torch.sigmoid(score)[:, None]
+        return out.to(h.dtype)
+
+
+@register_position("toy_learned_table")
+class ToyLearnedTable(PositionEncoding):
+    """Another family than rotary: a vector per position (here a fixed function of the position, so that no
+    parameter is needed), which the mixer that names it adds to its input."""
+
+    def vectors(self, positions, width):
+        j = torch.arange(width, device=positions.device, dtype=torch.float32)
+        return torch.sin(positions.float()[:, None] * (0.05 * (j + 1.0))[None, :]) * float(self.spec.amplitude)
+
+
+@register_mixer("toy_positional_sum")
+class ToyPositionalSum(Mixer):
+    """Running sum, per request, of (row + its position's vector): state of its own, and a position encoding
+    that is not rotary, chosen by the configuration."""
+
+    def __init__(self, spec):
+        super().__init__()
+        self.hidden = int(spec.hidden_size)
+        self.position = build_position(spec.position, self.hidden)
+
+    def param_specs(self):
+        return {}
+
+    def cache_need(self):
+        return CacheNeed(kv=None, state_shape=(self.hidden,), state_dtype=torch.float32)
+
+    def forward(self, h, ctx, cache):
+        x = h.float() + self.position.vectors(ctx.positions, self.hidden)
+        out = torch.empty_like(h)
+        slots, o = ctx.state_slots.tolist(), 0
+        for seg, n in enumerate(ctx.seg_lens):
+            run = cache.state[slots[seg]] + torch.cumsum(x[o:o + n], 0)
+            out[o:o + n] = (run / (ctx.positions[o:o + n].float() + 1.0)[:, None]).to(h.dtype)
+            cache.state[slots[seg]] = run[-1]
+            o += n
+        return out
+
+
+class ToyArchitectureTwo:
+    names = ("ToyTwoForCausalLM",)
+
+    def parse_config(self, top):
+        return dict(top)
+
+    def config_to_dict(self, cfg, architecture=None):
+        return dict(cfg)
+
+    def plan(self, cfg):
+        D = cfg["hidden_size"]
+        norm = part("rmsnorm", eps=1e-6, weighted=True, size=D)
+        layer = LayerSpec(mixer=part("toy_positional_sum", hidden_size=D,
+                                     position=part("toy_learned_table", amplitude=cfg["amplitude"])),
+                          feed_forward=part("toy_parity_experts", hidden_size=D),
+                          mixer_norm=norm, feed_forward_norm=norm)
+        return ModelPlan(vocab_size=cfg["vocab_size"], hidden_size=D, layers=(layer,),
+                         order=(OrderEntry(0, 0), OrderEntry(0, 1)), final_norm=norm)
+
+    def bindings(self, cfg, plan):
+        return []
+
+
+register_architecture(ToyArchitectureTwo())
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_toy_feed_forward_with_routing_and_toy_position_encoding(device):
+    """Registered, built from a plan and stepped like any other part; cutting and batching change nothing."""
+    from jax_llm_examples_amd.config import get_architecture
+    arch = get_architecture("ToyTwoForCausalLM")
+    cfg = arch.parse_config({"hidden_size": 40, "vocab_size": 61, "amplitude": 0.5})
+    model = DecoderModel(arch.plan(cfg), torch.float32, device)
+    model.allocate()
+    init_random_(model, seed=9, std=0.3)
+    assert isinstance(model.blocks[0].feed_forward, ToyParityExperts)
+    assert isinstance(model.blocks[0].mixer.position, ToyLearnedTable)
+    reqs = traces.random_requests(61, [37, 12, 29], seed=3)
+    results = {}
+    for mode in ("whole", "tail", "portions", "mixed"):
+        cache = CacheManager(model.cache_needs(), page_size=4, num_pages=8, max_requests=3, dtype=torch.float32,
+                             device=device)
+        assert cache.groups == [] and set(cache.state) == {0, 1}  # no pages at all: two runs with state
+        runner = ModelRunner(model, cache, _ops(device))
+        results[mode] = traces.run_trace(runner, getattr(traces, mode)(reqs))
+    for rid in reqs:
+        assert torch.isfinite(results["whole"][rid]).all()
+        for mode in ("tail", "portions", "mixed"):
+            assert torch.allclose(results[mode][rid], results["whole"][rid], rtol=1e-4, atol=1e-5), (mode, rid)
+    # both experts were used, and the position vectors matter
+    toks = reqs["r0"]
+    x = model.embed.params["weight"][torch.tensor(toks, device=device)].float()
+    h = P.rms_norm(x.cpu(), model.blocks[0].mixer_norm.params["weight"].cpu(), 1e-6)
+    assert 0 < int(((h @ model.blocks[0].feed_forward.params["direction"].cpu()) > 0).sum()) < len(toks) or len(toks) < 4
+    cfg0 = arch.parse_config({"hidden_size": 40, "vocab_size": 61, "amplitude": 0.0})
+    model0 = DecoderModel(arch.plan(cfg0), torch.float32, device)
+    model0.allocate()
+    init_random_(model0, seed=9, std=0.3)
+    cache = CacheManager(model0.cache_needs(), page_size=4, num_pages=8, max_requests=3, dtype=torch.float32,
+                         device=device)
+    other = traces.run_trace(ModelRunner(model0, cache, _ops(device)), traces.whole(reqs))
+    assert not torch.allclose(other["r0"], results["whole"]["r0"], rtol=1e-3, atol=1e-3)
 
 
 def test_order_is_checked():
