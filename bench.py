@@ -149,7 +149,8 @@ def main() -> int:
 
     achieved = nbytes["total"] / sec / 1e9
     out = {
-        "metric": "decode tok/s at batch 8, context 4096 (Llama 4 Scout layer sizes, random weights)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} "
+                  f"(Llama 4 {args.preset.split('-')[-1].capitalize()} layer sizes, random weights)",
         "value": round(args.batch / sec, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dkey,
