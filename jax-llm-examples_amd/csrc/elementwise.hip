@@ -132,6 +132,13 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
   __shared__ float red[THREADS / 64];
   const size_t n = blockIdx.x;
   const size_t base = n * D;
+  // (the weights are asked for first: they wait for nothing)
+  f32x4_t wv[CPT];
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int d = (threadIdx.x + THREADS * i) * 4;
+    wv[i] = (w != nullptr && d < D) ? load4<float>(w + d) : f32x4_t{1.f, 1.f, 1.f, 1.f};
+  }
   f32x4_t v[CPT];
   float ss = 0.f;
   const bool add = delta.any();
@@ -158,7 +165,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
     const int d = (threadIdx.x + THREADS * i) * 4;
     if (d < D) {
       f32x4_t h = v[i] * inv;
-      if (w != nullptr) h *= load4<float>(w + d);
+      if (w != nullptr) h *= wv[i];
       if (out != nullptr) store4<OT>(out + base + d, h);
       if (out32 != nullptr) store4<float>(out32 + base + d, h);
     }

@@ -27,22 +27,32 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const float* __restrict
     for (int j = 0; j < EPW; ++j) acc[t][j] = 0.f;
   if (VEC) {  // D is a multiple of 4: rows are 16-byte aligned
     const int D4 = D >> 2;
-#pragma unroll 2
-    for (int c = lane; c < D4; c += 64) {
-      float4 wv[EPW];
+    // U chunks are loaded before any is used (a lone wavefront would otherwise wait for memory once per chunk);
+    // chunks past the row's end are loaded from its last chunk and count as zeros
+    constexpr int U = TPB * EPW == 1 ? 8 : 2;
+    for (int c0 = lane; c0 < D4; c0 += 64 * U) {
+      float4 wv[U][EPW], xv[U][TPB];
 #pragma unroll
-      for (int j = 0; j < EPW; ++j) wv[j] = *reinterpret_cast<const float4*>(we[j] + 4 * c);
+      for (int u = 0; u < U; ++u) {
+        const int c = min(c0 + 64 * u, D4 - 1);
 #pragma unroll
-      for (int t = 0; t < TPB; ++t) {
-        if (n0 + t < N) {
-          const float4 xv = *reinterpret_cast<const float4*>(h + (size_t)(n0 + t) * D + 4 * c);
+        for (int j = 0; j < EPW; ++j) wv[u][j] = *reinterpret_cast<const float4*>(we[j] + 4 * c);
 #pragma unroll
-          for (int j = 0; j < EPW; ++j) {
-            acc[t][j] += xv.x * wv[j].x;
-            acc[t][j] += xv.y * wv[j].y;
-            acc[t][j] += xv.z * wv[j].z;
-            acc[t][j] += xv.w * wv[j].w;
-          }
+        for (int t = 0; t < TPB; ++t)
+          xv[u][t] = *reinterpret_cast<const float4*>(h + (size_t)min(n0 + t, N - 1) * D + 4 * c);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (c0 + 64 * u < D4) {
+#pragma unroll
+          for (int t = 0; t < TPB; ++t)
+#pragma unroll
+            for (int j = 0; j < EPW; ++j) {
+              acc[t][j] += xv[u][t].x * wv[u][j].x;
+              acc[t][j] += xv[u][t].y * wv[u][j].y;
+              acc[t][j] += xv[u][t].z * wv[u][j].z;
+              acc[t][j] += xv[u][t].w * wv[u][j].w;
+            }
         }
       }
     }
@@ -66,13 +76,10 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const float* __restrict
     }
 }
 
-// The k largest logits of each token (lowest index first among equals) and their sigmoids.
-__global__ void moe_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids, float* __restrict__ gates,
-                                int N, int E, int k) {
-  const size_t n = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (n >= (size_t)N) return;
+// The k largest logits of token n (lowest index first among equals) and their sigmoids.
+__device__ __forceinline__ void topk_of_token(const float* __restrict__ logits, size_t n, int E, int k,
+                                              int (&best_i)[kMaxTopK], float (&gate)[kMaxTopK]) {
   float best_v[kMaxTopK];
-  int best_i[kMaxTopK];
 #pragma unroll
   for (int j = 0; j < kMaxTopK; ++j) {
     best_v[j] = -INFINITY;
@@ -98,49 +105,33 @@ __global__ void moe_topk_kernel(const float* __restrict__ logits, int* __restric
     }
   }
 #pragma unroll
+  for (int j = 0; j < kMaxTopK; ++j) gate[j] = 1.0f / (1.0f + expf(-best_v[j]));
+}
+
+__global__ void moe_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids, float* __restrict__ gates,
+                                int N, int E, int k) {
+  const size_t n = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= (size_t)N) return;
+  int best_i[kMaxTopK];
+  float gate[kMaxTopK];
+  topk_of_token(logits, n, E, k, best_i, gate);
+#pragma unroll
   for (int j = 0; j < kMaxTopK; ++j) {
     if (j < k) {
       ids[n * k + j] = best_i[j];
-      gates[n * k + j] = 1.0f / (1.0f + expf(-best_v[j]));
+      gates[n * k + j] = gate[j];
     }
   }
 }
 
-// logits: [N, E] float32 workspace (also the caller's copy of the router logits)
-JLE_API int jle_moe_route(const float* h, const float* w, int* ids, float* gates, float* logits, int N, int D, int E,
-                          int k, hipStream_t s) {
-  if (N <= 0) return 0;
-  if (k < 1 || k > kMaxTopK || k > E || E > 4096 || logits == nullptr) return JLE_BAD_ARG;
-  const bool vec = D % 4 == 0 && (((uintptr_t)h | (uintptr_t)w) & 15) == 0;
-  // few rows: a wavefront per (token, expert) keeps more of them in flight; many: a wavefront takes 2 tokens
-  // and 4 experts, so that the rows of h are read 4 times less often
-  const bool many = N >= 512;
-  dim3 b(256);
-  if (many) {
-    dim3 g((N + 1) / 2, (E + 15) / 16);
-    if (vec) hipLaunchKernelGGL((moe_logits_kernel<2, 4, true>), g, b, 0, s, h, w, logits, N, D, E);
-    else hipLaunchKernelGGL((moe_logits_kernel<2, 4, false>), g, b, 0, s, h, w, logits, N, D, E);
-  } else {
-    dim3 g(N, (E + 3) / 4);
-    if (vec) hipLaunchKernelGGL((moe_logits_kernel<1, 1, true>), g, b, 0, s, h, w, logits, N, D, E);
-    else hipLaunchKernelGGL((moe_logits_kernel<1, 1, false>), g, b, 0, s, h, w, logits, N, D, E);
-  }
-  JLE_LAUNCH_CHECK();
-  hipLaunchKernelGGL(moe_topk_kernel, dim3((N + 127) / 128), dim3(128), 0, s, logits, ids, gates, N, E, k);
-  JLE_LAUNCH_CHECK();
-  return 0;
-}
-
-// Stable counting sort of the M = N * k pairs by expert, one block.
+// Stable counting sort of the M = N * k pairs by expert, by one block.
 //   offsets[e] .. offsets[e + 1]: rows of expert e in sorted order
 //   sorted_token[s]: the token of sorted row s;  sorted_gate[s]: its gate;  inv[r]: sorted row of pair r
-__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, const float* __restrict__ gates,
-                                                         int* __restrict__ offsets, int* __restrict__ sorted_token,
-                                                         float* __restrict__ sorted_gate, int* __restrict__ inv,
-                                                         int M, int E, int k) {
-  extern __shared__ int smem[];  // counts[E] then starts[E + 1]
-  int* counts = smem;
-  int* starts = smem + E;
+// ids and gates may lie in shared memory; counts[E] and starts[E + 1] do.
+__device__ __forceinline__ void align_by_block(const int* ids, const float* gates, int* counts, int* starts,
+                                               int* __restrict__ offsets, int* __restrict__ sorted_token,
+                                               float* __restrict__ sorted_gate, int* __restrict__ inv, int M, int E,
+                                               int k) {
   for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
   __syncthreads();
   for (int r = threadIdx.x; r < M; r += blockDim.x) atomicAdd(&counts[ids[r]], 1);
@@ -174,12 +165,104 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__
   }
 }
 
-JLE_API int jle_moe_align(const int* ids, const float* gates, int* offsets, int* sorted_token, float* sorted_gate,
-                          int* inv, int M, int E, int k, hipStream_t s) {
-  if (M <= 0) return 0;
-  if (E < 1 || E > 4096) return JLE_BAD_ARG;
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, const float* __restrict__ gates,
+                                                         int* __restrict__ offsets, int* __restrict__ sorted_token,
+                                                         float* __restrict__ sorted_gate, int* __restrict__ inv,
+                                                         int M, int E, int k) {
+  extern __shared__ int smem[];  // counts[E] then starts[E + 1]
+  align_by_block(ids, gates, smem, smem + E, offsets, sorted_token, sorted_gate, inv, M, E, k);
+}
+
+// Both in one block, for steps of few tokens (N <= 1024): thread n chooses for token n and leaves its pairs in
+// shared memory, from where the block groups them.
+__global__ __launch_bounds__(1024) void moe_topk_align_kernel(const float* __restrict__ logits, int* __restrict__ ids,
+                                                              float* __restrict__ gates, int* __restrict__ offsets,
+                                                              int* __restrict__ sorted_token,
+                                                              float* __restrict__ sorted_gate, int* __restrict__ inv,
+                                                              int N, int E, int k) {
+  extern __shared__ int smem[];  // counts[E], starts[E + 1], ids[N * k], gates[N * k]
+  const int M = N * k;
+  int* ids_s = smem + 2 * E + 1;
+  float* gates_s = reinterpret_cast<float*>(ids_s + M);
+  const int n = threadIdx.x;
+  if (n < N) {
+    int best_i[kMaxTopK];
+    float gate[kMaxTopK];
+    topk_of_token(logits, (size_t)n, E, k, best_i, gate);
+#pragma unroll
+    for (int j = 0; j < kMaxTopK; ++j) {
+      if (j < k) {
+        ids[n * k + j] = best_i[j];
+        gates[n * k + j] = gate[j];
+        ids_s[n * k + j] = best_i[j];
+        gates_s[n * k + j] = gate[j];
+      }
+    }
+  }
+  __syncthreads();
+  align_by_block(ids_s, gates_s, smem, smem + E, offsets, sorted_token, sorted_gate, inv, M, E, k);
+}
+
+static int launch_logits(const float* h, const float* w, float* logits, int N, int D, int E, hipStream_t s) {
+  const bool vec = D % 4 == 0 && (((uintptr_t)h | (uintptr_t)w) & 15) == 0;
+  // few rows: a wavefront per (token, expert) keeps more of them in flight; many: a wavefront takes 2 tokens
+  // and 4 experts, so that the rows of h are read 4 times less often
+  const bool many = N >= 512;
+  dim3 b(256);
+  if (many) {
+    dim3 g((N + 1) / 2, (E + 15) / 16);
+    if (vec) hipLaunchKernelGGL((moe_logits_kernel<2, 4, true>), g, b, 0, s, h, w, logits, N, D, E);
+    else hipLaunchKernelGGL((moe_logits_kernel<2, 4, false>), g, b, 0, s, h, w, logits, N, D, E);
+  } else {
+    dim3 g(N, (E + 3) / 4);
+    if (vec) hipLaunchKernelGGL((moe_logits_kernel<1, 1, true>), g, b, 0, s, h, w, logits, N, D, E);
+    else hipLaunchKernelGGL((moe_logits_kernel<1, 1, false>), g, b, 0, s, h, w, logits, N, D, E);
+  }
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
+static int launch_align(const int* ids, const float* gates, int* offsets, int* sorted_token, float* sorted_gate,
+                        int* inv, int M, int E, int k, hipStream_t s) {
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (2 * E + 1) * sizeof(int), s, ids, gates, offsets,
                      sorted_token, sorted_gate, inv, M, E, k);
   JLE_LAUNCH_CHECK();
   return 0;
+}
+
+// logits: [N, E] float32 workspace (also the caller's copy of the router logits)
+JLE_API int jle_moe_route(const float* h, const float* w, int* ids, float* gates, float* logits, int N, int D, int E,
+                          int k, hipStream_t s) {
+  if (N <= 0) return 0;
+  if (k < 1 || k > kMaxTopK || k > E || E > 4096 || logits == nullptr) return JLE_BAD_ARG;
+  if (int rc = launch_logits(h, w, logits, N, D, E, s)) return rc;
+  hipLaunchKernelGGL(moe_topk_kernel, dim3((N + 127) / 128), dim3(128), 0, s, logits, ids, gates, N, E, k);
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
+// The router and the grouping of its choices in one call (the same results as jle_moe_route, then jle_moe_align).
+JLE_API int jle_moe_route_align(const float* h, const float* w, int* ids, float* gates, float* logits, int* offsets,
+                                int* sorted_token, float* sorted_gate, int* inv, int N, int D, int E, int k,
+                                hipStream_t s) {
+  if (N <= 0) return 0;
+  if (k < 1 || k > kMaxTopK || k > E || E > 4096 || logits == nullptr) return JLE_BAD_ARG;
+  if (int rc = launch_logits(h, w, logits, N, D, E, s)) return rc;
+  const size_t words = (size_t)2 * E + 1 + (size_t)2 * N * k;
+  if (N <= 1024 && words <= 12000) {
+    hipLaunchKernelGGL(moe_topk_align_kernel, dim3(1), dim3(1024), words * sizeof(int), s, logits, ids, gates,
+                       offsets, sorted_token, sorted_gate, inv, N, E, k);
+    JLE_LAUNCH_CHECK();
+    return 0;
+  }
+  hipLaunchKernelGGL(moe_topk_kernel, dim3((N + 127) / 128), dim3(128), 0, s, logits, ids, gates, N, E, k);
+  JLE_LAUNCH_CHECK();
+  return launch_align(ids, gates, offsets, sorted_token, sorted_gate, inv, N * k, E, k, s);
+}
+
+JLE_API int jle_moe_align(const int* ids, const float* gates, int* offsets, int* sorted_token, float* sorted_gate,
+                          int* inv, int M, int E, int k, hipStream_t s) {
+  if (M <= 0) return 0;
+  if (E < 1 || E > 4096) return JLE_BAD_ARG;
+  return launch_align(ids, gates, offsets, sorted_token, sorted_gate, inv, M, E, k, s);
 }

@@ -28,6 +28,7 @@ _SIGNATURES = {
     "jle_paged_attention_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _vp],
     "jle_moe_route": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "jle_moe_route_align": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
@@ -428,16 +429,29 @@ class HipOps:
         return out
 
     # ------------------------------------------------------------------ routed experts
-    def moe_route(self, h32, router, top_k: int, want_logits: bool = False):
+    def moe_route(self, h32, router, top_k: int, want_logits: bool = False, group: bool = False):
+        """``group``: also return the grouping of the choices by expert (what ``moe_align`` gives), made in
+        the same call; ``moe_experts`` takes it as ``grouping``."""
         n, d = h32.shape
         e = router.shape[0]
         self._chk(h32, torch.float32, None, "router input")
         self._chk(router, torch.float32, (e, d), "router matrix")
         if not 1 <= top_k <= min(8, e) or e > 4096:
             raise KernelError(f"router kernel: top_k {top_k} of {e} experts is not supported (top_k <= 8, experts <= 4096)")
-        ids = torch.empty(n, top_k, dtype=torch.int32, device=h32.device)
-        gates = torch.empty(n, top_k, dtype=torch.float32, device=h32.device)
-        logits = torch.empty(n, e, dtype=torch.float32, device=h32.device)
+        dev = h32.device
+        ids = torch.empty(n, top_k, dtype=torch.int32, device=dev)
+        gates = torch.empty(n, top_k, dtype=torch.float32, device=dev)
+        logits = torch.empty(n, e, dtype=torch.float32, device=dev)
+        if group:
+            m = n * top_k
+            offsets = torch.empty(e + 1, dtype=torch.int32, device=dev)
+            sorted_token = torch.empty(m, dtype=torch.int32, device=dev)
+            sorted_gate = torch.empty(m, dtype=torch.float32, device=dev)
+            inv = torch.empty(m, dtype=torch.int32, device=dev)
+            self._call("jle_moe_route_align", _p(h32), _p(router), _p(ids), _p(gates), _p(logits), _p(offsets),
+                       _p(sorted_token), _p(sorted_gate), _p(inv), n, d, e, top_k)
+            grouping = (offsets, sorted_token, sorted_gate, inv)
+            return (ids, gates, logits, grouping) if want_logits else (ids, gates, grouping)
         self._call("jle_moe_route", _p(h32), _p(router), _p(ids), _p(gates), _p(logits), n, d, e, top_k)
         return (ids, gates, logits) if want_logits else (ids, gates)
 
@@ -455,11 +469,13 @@ class HipOps:
                    m, num_experts, k)
         return offsets, sorted_token, sorted_gate, inv
 
-    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False):
+    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None):
         n, d = h.shape
         e, f2, _ = w_gate_up.shape
         k = expert_ids.shape[1]
-        offsets, sorted_token, sorted_gate, inv = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e)
+        if grouping is None:
+            grouping = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e)
+        offsets, sorted_token, sorted_gate, inv = grouping
         mfma = h.dtype == torch.bfloat16 and d % 8 == 0 and (f2 // 2) % 8 == 0
         if mfma and n * k <= 2 * self.SKINNY_MAX_ROWS:  # few rows: the cost is streaming the chosen experts' weights
             act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,

@@ -156,16 +156,18 @@ class ReferenceOps:
         return out
 
     # ------------------------------------------------------------------ routed experts
-    def moe_route(self, h32, router, top_k: int):
+    def moe_route(self, h32, router, top_k: int, group: bool = False):
         """Router logits in float32, the ``top_k`` largest per token (lowest index
-        first among equals), gate = sigmoid of the chosen logit."""
+        first among equals), gate = sigmoid of the chosen logit.  ``group``: a third result, the
+        grouping of the choices by expert for ``moe_experts`` (none here: these ops do not group)."""
         logits = h32.float() @ router.float().t()
         # stable sort by (-logit, index): lowest index wins ties
         order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :top_k]
         vals = torch.gather(logits, 1, order)
-        return order.to(torch.int32), torch.sigmoid(vals)
+        ids, gates = order.to(torch.int32), torch.sigmoid(vals)
+        return (ids, gates, None) if group else (ids, gates)
 
-    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False):
+    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None):
         """``sum_j  W_down[e_j] (silu(g_j W_gate[e_j] h) * (g_j W_up[e_j] h))`` per token,
         plus ``shared`` if given; float32 result.  ``w_gate_up`` is ``[E, 2F, D]`` (gate rows then
         up rows), ``w_down`` ``[E, D, F]``.  Activations between the two products are

@@ -71,14 +71,15 @@ class MoESigmoidShared(FeedForward):
 
     def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
         ops = ctx.ops
-        expert_ids, gates = ops.moe_route(h32, self.params["router"], self.top_k)
+        expert_ids, gates, grouping = ops.moe_route(h32, self.params["router"], self.top_k, group=True)
         if ctx.record_routing:
             self.last_routing = (expert_ids.clone(), gates.clone())
         forced = ctx.forced_routing.get(id(self)) if ctx.forced_routing else None
         if forced is not None:
             expert_ids, gates = forced
+            grouping = None
         shared = None
         if self.shared_inter:
             shared = ops.linear(ops.swiglu_linear(h, self.params["shared_gate_up"]), self.params["shared_down"])
         return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"], shared,
-                               tiled=self.tiled)
+                               tiled=self.tiled, grouping=grouping)

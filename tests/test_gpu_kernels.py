@@ -271,6 +271,20 @@ def test_router_logits_of_a_token_do_not_depend_on_the_batch(ops, n, d, e, k):
         assert torch.equal(l2, logits[lo:hi]) and torch.equal(i2, ids[lo:hi]) and torch.equal(g2, gates[lo:hi])
 
 
+@pytest.mark.parametrize("n,d,e,k", [(1, 64, 16, 1), (8, 5120, 16, 1), (64, 96, 128, 2), (1000, 80, 5, 3), (1024, 64, 9, 8),
+                                     (1025, 64, 7, 2), (900, 64, 4000, 1), (3000, 72, 16, 1)])
+def test_router_and_grouping_in_one_call(ops, n, d, e, k):
+    """Few tokens: one block chooses and groups; many tokens, or tables too long for its shared memory: the separate
+    kernels.  Either way the same as route, then align."""
+    h, w = _rand(n, d, seed=1), _rand(e, d, scale=0.05, seed=2)
+    ids, gates, logits = ops.moe_route(h, w, k, want_logits=True)
+    want = ops.moe_align(ids, gates, e)
+    ids2, gates2, logits2, grouping = ops.moe_route(h, w, k, want_logits=True, group=True)
+    assert torch.equal(ids, ids2) and torch.equal(gates, gates2) and torch.equal(logits, logits2)
+    for a, b in zip(want, grouping):
+        assert torch.equal(a, b)
+
+
 def test_moe_route_lowest_index_wins_ties(ops):
     h = _rand(5, 64, seed=1)
     w = _rand(1, 64, seed=2).expand(6, 64).contiguous()  # every expert the same score
