@@ -18,7 +18,7 @@ from plain_llama4 import PlainModel
 from tiny_configs import FAST, TINY, write_tiny
 
 LENGTHS = {"A": [1, 80, 33, 47, 64, 9], "B": [120, 2, 49, 96, 31, 77], "C": [61, 40, 5, 83], "D": [37, 70, 3, 55, 64, 21],
-           "F": [300, 40, 170, 33]}
+           "F": [300, 40, 170, 33], "W": [700, 33, 260, 48]}
 MODES = {"whole": traces.whole, "tail": traces.tail, "portions": traces.portions, "mixed": traces.mixed}
 TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}  # of the largest logit of the request
 
@@ -28,7 +28,7 @@ def _vocab(name):
     return c.get("text_config", c)["vocab_size"]
 
 
-def _check(name, folder, dtype, device, mode, reference_ops):
+def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu"):
     lengths = LENGTHS[name] + (LENGTHS[name][::-1] + LENGTHS[name] if mode == "mixed" else [])
     reqs = traces.random_requests(_vocab(name), lengths, seed=5)
     steps = MODES[mode](reqs)
@@ -40,11 +40,23 @@ def _check(name, folder, dtype, device, mode, reference_ops):
     runner.cache.check()
     assert runner.cache.num_live() == 0 and all(g.pool.num_held == 0 for g in runner.cache.groups)
     plain = PlainModel(folder)
+    if plain_device != "cpu":  # (plain PyTorch all the same; the wide configuration would take minutes on the CPU)
+        plain.w = {k: v.to(plain_device) for k, v in plain.w.items()}
     worst = 0.0
     for rid, toks in reqs.items():
         forced = routes.get(rid) if dtype == "bfloat16" else None
         info = {}
-        ref = plain.logits(toks, forced=forced, info=info)
+        if plain_device != "cpu":
+            prev = torch.get_default_device()
+            torch.set_default_device(plain_device)
+            try:
+                forced = {li: ids.to(plain_device) for li, ids in forced.items()} if forced else forced
+                ref = plain.logits(toks, forced=forced, info=info).cpu()
+                info = {li: (idx.cpu(), sc.cpu()) for li, (idx, sc) in info.items()}
+            finally:
+                torch.set_default_device(prev)
+        else:
+            ref = plain.logits(toks, forced=forced, info=info)
         assert got[rid].shape == ref.shape
         assert torch.isfinite(got[rid]).all(), f"{rid}: non-finite logits (a page that was given back?)"
         err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
@@ -99,6 +111,25 @@ def test_gpu_bfloat16_sizes_of_the_fast_kernels(tmp_path_factory, mode, monkeypa
     _check("F", folder, "bfloat16", "cuda:0", mode, reference_ops=False)
     if mode in ("whole", "tail"):  # the other modes cut the prompts into portions too short for it
         assert calls["stream"] > 0, "no step went through the weight-streaming grouped product"
+
+
+@pytest.fixture(scope="module")
+def wide_model_dir(tmp_path_factory):
+    return write_tiny("W", str(tmp_path_factory.mktemp("models_wide") / "W"), torch.bfloat16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+def test_gpu_bfloat16_serving_widths(wide_model_dir, mode):
+    """Two layers (one rotary, one without) at the widths the benchmark runs: the kernel variants that only these
+    sizes reach (rows of 5120, 40 heads on 8, experts 8192 wide) against the plain implementation."""
+    _check("W", wide_model_dir, "bfloat16", "cuda:0", mode, reference_ops=False, plain_device="cuda:0")
+
+
+@pytest.mark.gpu
+def test_gpu_float32_serving_widths(tmp_path):
+    folder = write_tiny("W", str(tmp_path / "W32"), torch.float32)
+    _check("W", folder, "float32", "cuda:0", "mixed", reference_ops=False, plain_device="cuda:0")
 
 
 @pytest.mark.gpu

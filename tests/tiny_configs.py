@@ -71,6 +71,21 @@ FAST = {
     },
 }
 
+# The widths that serving runs at (Llama 4 Scout's: width 5120, 40 query heads on 8 kv heads of 128, experts 8192
+# wide, chunk 8192 and its frequency scaling), with few layers, few experts and a short vocabulary that is no
+# power of two: about 3 GB in bfloat16 (GPU tests only)
+FAST["W"] = {
+    "architectures": ["Llama4ForCausalLM"],
+    "seed": 67,
+    "num_hidden_layers": 2, "hidden_size": 5120, "num_attention_heads": 40, "num_key_value_heads": 8,
+    "head_dim": 128, "interleave_moe_layer_step": 1, "num_local_experts": 4, "num_experts_per_tok": 1,
+    "intermediate_size": 8192, "intermediate_size_mlp": 16384, "vocab_size": 20008, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 16.0, "low_freq_factor": 1.0, "high_freq_factor": 1.0,
+                     "original_max_position_embeddings": 8192},
+    "no_rope_layers": [1, 0], "attention_chunk_size": 8192, "use_qk_norm": True, "attn_temperature_tuning": True,
+    "floor_scale": 8192, "attn_scale": 0.1, "rms_norm_eps": 1e-5, "tie_word_embeddings": False,
+}
+
 
 def tiny_config_json(name: str) -> dict:
     c = {k: v for k, v in {**TINY, **FAST}[name].items() if k != "seed"}
