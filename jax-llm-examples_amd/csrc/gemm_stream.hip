@@ -45,8 +45,9 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, float b, floa
   *reinterpret_cast<uint2*>(p) = uint2{pack_bf16(a, b), pack_bf16(c, d)};
 }
 
-// The work of one block once it knows its rows and tiles; NTL = B tiles (of 16 rows) that hold live rows, a
-// multiple of 4.  The main loop has no branch but its own: every load is asked for unconditionally (rows past
+// The work of one block once it knows its rows and tiles; NTL = B tiles (of 16 rows) that hold live rows, even
+// (the rows are brought in by whole rounds of the block's threads, 64 rows each: a round's rows past the live
+// tiles land in tiles that nobody reads).  The main loop has no branch but its own: every load is asked for unconditionally (rows past
 // the live ones read the pass's first row again, into their own places), so that the waits for the loads of
 // two stages ago never include the loads asked for since.
 template <bool SWIGLU, typename OutT, int WAVES, int NTL>
@@ -216,12 +217,15 @@ __global__ __launch_bounds__(WAVES * 64, 2) void gemm_stream_kernel(const bf16_t
   }
   const bf16_t* w0 = We + (size_t)t0 * nkb * 512 + lane * 8;
   const bf16_t* w1 = We + (size_t)t1 * nkb * 512 + lane * 8;
-  if (live <= 64)
-    stream_block<SWIGLU, OutT, WAVES, 4>(X, w0, w1, Y, a_rows, scale, sX, tok0, live, K, Nout, t0, t1, wave_ok);
-  else if (live <= 128)
-    stream_block<SWIGLU, OutT, WAVES, 8>(X, w0, w1, Y, a_rows, scale, sX, tok0, live, K, Nout, t0, t1, wave_ok);
-  else
-    stream_block<SWIGLU, OutT, WAVES, 12>(X, w0, w1, Y, a_rows, scale, sX, tok0, live, K, Nout, t0, t1, wave_ok);
+#define GO(NTL_) \
+  stream_block<SWIGLU, OutT, WAVES, NTL_>(X, w0, w1, Y, a_rows, scale, sX, tok0, live, K, Nout, t0, t1, wave_ok)
+  if (live <= 32) GO(2);
+  else if (live <= 64) GO(4);
+  else if (live <= 96) GO(6);
+  else if (live <= 128) GO(8);
+  else if (live <= 160) GO(10);
+  else GO(12);
+#undef GO
 }
 
 template <bool SW, typename OT, int WV>
