@@ -43,7 +43,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                                                           OutT* __restrict__ Y, const int* __restrict__ offsets,
                                                           const int* __restrict__ a_rows,
                                                           const float* __restrict__ scale, int M, int Nout, int K,
-                                                          int tiled) {
+                                                          int tiled, const bf16_t* __restrict__ W_last,
+                                                          int tiled_last) {
   static_assert(RT == 2 || !SWIGLU, "the fused activation needs the gate tile and the up tile");
   __shared__ float red[WAVES][RT * MT * 4][64];
   const int e = blockIdx.z;
@@ -57,6 +58,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int r = lane & 15, g = lane >> 4;
   const bf16_t* We = W + (size_t)e * Nout * K;
+  if (W_last != nullptr && e == (int)gridDim.z - 1) {  // the last group's matrix lies elsewhere (a shared expert)
+    We = W_last;
+    tiled = tiled_last;
+  }
   const int half = Nout >> 1;
   const int base = SWIGLU ? blockIdx.x * 16 : blockIdx.x * (16 * RT);  // first output column of the block
   int ra0, ra1;  // the weight rows this lane reads
@@ -168,12 +173,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 template <int MT, bool SW, typename OT>
 static int launch_skinny(int xrows, int ytiles, int G, hipStream_t s, int variant, const void* X, const void* W,
                          void* Y, const int* offsets, const int* a_rows, const float* scale, int M, int Nout, int K,
-                         int tiled) {
+                         int tiled, const void* W_last, int tiled_last) {
 #define LAUNCH(RT, WV, UN)                                                                                       \
   do {                                                                                                           \
     dim3 g((xrows + 16 * (SW ? 1 : RT) - 1) / (16 * (SW ? 1 : RT)), ytiles, G);                                  \
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, SW, OT, WV, UN, (SW ? 2 : RT)>), g, dim3(WV * 64), 0, s,          \
-                       (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, offsets, a_rows, scale, M, Nout, K, tiled);   \
+                       (const bf16_t*)X, (const bf16_t*)W, (OT*)Y, offsets, a_rows, scale, M, Nout, K, tiled,    \
+                       (const bf16_t*)W_last, tiled_last);                                                       \
     return 0;                                                                                                    \
   } while (0)
   switch (variant) {
@@ -192,10 +198,14 @@ static int launch_skinny(int xrows, int ytiles, int G, hipStream_t s, int varian
 
 // X [*, K] bf16, W [G, Nout, K] bf16, Y [M, Nout] (or [M, Nout / 2] with swiglu) bf16 or float32.
 // max_rows: the most rows any group can have (M if unknown).  variant: 0 = chosen from the sizes.
+// W_last: if given, the matrix of the last of the G groups (W then holds G - 1), row-major or in the streaming
+// layout by tiled_last: a shared expert's rows go through the same launch as the routed experts'.
 JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* offsets, const int* a_rows,
                             const float* scale, int swiglu, int out_f32, int M, int Nout, int K, int G, int max_rows,
-                            int variant, int tiled, hipStream_t s) {
+                            int variant, int tiled, const void* W_last, int tiled_last, hipStream_t s) {
   if (M <= 0 || Nout <= 0) return 0;
+  if (W_last != nullptr && (offsets == nullptr || G < 2)) return JLE_BAD_ARG;
+  if (W_last != nullptr && tiled_last && (K % 32 || Nout % 16 || (swiglu && (Nout / 2) % 16))) return JLE_BAD_ARG;
   if (K <= 0 || K % 8 || G < 1 || G > 65535 || (swiglu && Nout % 2)) return JLE_BAD_ARG;
   if (tiled && (K % 32 || Nout % 16 || (swiglu && (Nout / 2) % 16))) return JLE_BAD_ARG;
   if (max_rows <= 0 || max_rows > M) max_rows = M;
@@ -214,9 +224,9 @@ JLE_API int jle_gemm_skinny(const void* X, const void* W, void* Y, const int* of
   int rc;
 #define PICK(SW, OT)                                                                                             \
   do {                                                                                                           \
-    if (mt == 1) rc = launch_skinny<1, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled);      \
-    else if (mt == 2) rc = launch_skinny<2, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled); \
-    else rc = launch_skinny<4, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled);              \
+    if (mt == 1) rc = launch_skinny<1, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last);      \
+    else if (mt == 2) rc = launch_skinny<2, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last); \
+    else rc = launch_skinny<4, SW, OT>(xrows, ytiles, G, s, variant, X, W, Y, offsets, a_rows, scale, M, Nout, K, tiled, W_last, tiled_last);              \
   } while (0)
   if (swiglu) {
     if (out_f32) PICK(true, float); else PICK(true, bf16_t);

@@ -128,10 +128,19 @@ __global__ void moe_topk_kernel(const float* __restrict__ logits, int* __restric
 //   offsets[e] .. offsets[e + 1]: rows of expert e in sorted order
 //   sorted_token[s]: the token of sorted row s;  sorted_gate[s]: its gate;  inv[r]: sorted row of pair r
 // ids and gates may lie in shared memory; counts[E] and starts[E + 1] do.
+// extra > 0: one more group behind the experts' that holds every token once, in order, with gate 1
+// (offsets[E + 1] = M + extra; rows M .. M + extra - 1): the rows of a shared expert.
 __device__ __forceinline__ void align_by_block(const int* ids, const float* gates, int* counts, int* starts,
                                                int* __restrict__ offsets, int* __restrict__ sorted_token,
                                                float* __restrict__ sorted_gate, int* __restrict__ inv, int M, int E,
-                                               int k) {
+                                               int k, int extra) {
+  if (extra > 0) {
+    if (threadIdx.x == 0) offsets[E + 1] = M + extra;
+    for (int i = threadIdx.x; i < extra; i += blockDim.x) {
+      sorted_token[M + i] = i;
+      sorted_gate[M + i] = 1.0f;
+    }
+  }
   for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
   __syncthreads();
   for (int r = threadIdx.x; r < M; r += blockDim.x) atomicAdd(&counts[ids[r]], 1);
@@ -168,9 +177,9 @@ __device__ __forceinline__ void align_by_block(const int* ids, const float* gate
 __global__ __launch_bounds__(1024) void moe_align_kernel(const int* __restrict__ ids, const float* __restrict__ gates,
                                                          int* __restrict__ offsets, int* __restrict__ sorted_token,
                                                          float* __restrict__ sorted_gate, int* __restrict__ inv,
-                                                         int M, int E, int k) {
+                                                         int M, int E, int k, int extra) {
   extern __shared__ int smem[];  // counts[E] then starts[E + 1]
-  align_by_block(ids, gates, smem, smem + E, offsets, sorted_token, sorted_gate, inv, M, E, k);
+  align_by_block(ids, gates, smem, smem + E, offsets, sorted_token, sorted_gate, inv, M, E, k, extra);
 }
 
 // Both in one block, for steps of few tokens (N <= 1024): thread n chooses for token n and leaves its pairs in
@@ -179,7 +188,7 @@ __global__ __launch_bounds__(1024) void moe_topk_align_kernel(const float* __res
                                                               float* __restrict__ gates, int* __restrict__ offsets,
                                                               int* __restrict__ sorted_token,
                                                               float* __restrict__ sorted_gate, int* __restrict__ inv,
-                                                              int N, int E, int k) {
+                                                              int N, int E, int k, int extra) {
   extern __shared__ int smem[];  // counts[E], starts[E + 1], ids[N * k], gates[N * k]
   const int M = N * k;
   int* ids_s = smem + 2 * E + 1;
@@ -200,7 +209,7 @@ __global__ __launch_bounds__(1024) void moe_topk_align_kernel(const float* __res
     }
   }
   __syncthreads();
-  align_by_block(ids_s, gates_s, smem, smem + E, offsets, sorted_token, sorted_gate, inv, M, E, k);
+  align_by_block(ids_s, gates_s, smem, smem + E, offsets, sorted_token, sorted_gate, inv, M, E, k, extra);
 }
 
 static int launch_logits(const float* h, const float* w, float* logits, int N, int D, int E, hipStream_t s) {
@@ -223,9 +232,9 @@ static int launch_logits(const float* h, const float* w, float* logits, int N, i
 }
 
 static int launch_align(const int* ids, const float* gates, int* offsets, int* sorted_token, float* sorted_gate,
-                        int* inv, int M, int E, int k, hipStream_t s) {
+                        int* inv, int M, int E, int k, int extra, hipStream_t s) {
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (2 * E + 1) * sizeof(int), s, ids, gates, offsets,
-                     sorted_token, sorted_gate, inv, M, E, k);
+                     sorted_token, sorted_gate, inv, M, E, k, extra);
   JLE_LAUNCH_CHECK();
   return 0;
 }
@@ -242,27 +251,28 @@ JLE_API int jle_moe_route(const float* h, const float* w, int* ids, float* gates
 }
 
 // The router and the grouping of its choices in one call (the same results as jle_moe_route, then jle_moe_align).
+// extra_group: offsets has E + 2 entries, sorted_token and sorted_gate N * k + N (see align_by_block).
 JLE_API int jle_moe_route_align(const float* h, const float* w, int* ids, float* gates, float* logits, int* offsets,
                                 int* sorted_token, float* sorted_gate, int* inv, int N, int D, int E, int k,
-                                hipStream_t s) {
+                                int extra_group, hipStream_t s) {
   if (N <= 0) return 0;
   if (k < 1 || k > kMaxTopK || k > E || E > 4096 || logits == nullptr) return JLE_BAD_ARG;
   if (int rc = launch_logits(h, w, logits, N, D, E, s)) return rc;
   const size_t words = (size_t)2 * E + 1 + (size_t)2 * N * k;
   if (N <= 1024 && words <= 12000) {
     hipLaunchKernelGGL(moe_topk_align_kernel, dim3(1), dim3(1024), words * sizeof(int), s, logits, ids, gates,
-                       offsets, sorted_token, sorted_gate, inv, N, E, k);
+                       offsets, sorted_token, sorted_gate, inv, N, E, k, extra_group ? N : 0);
     JLE_LAUNCH_CHECK();
     return 0;
   }
   hipLaunchKernelGGL(moe_topk_kernel, dim3((N + 127) / 128), dim3(128), 0, s, logits, ids, gates, N, E, k);
   JLE_LAUNCH_CHECK();
-  return launch_align(ids, gates, offsets, sorted_token, sorted_gate, inv, N * k, E, k, s);
+  return launch_align(ids, gates, offsets, sorted_token, sorted_gate, inv, N * k, E, k, extra_group ? N : 0, s);
 }
 
 JLE_API int jle_moe_align(const int* ids, const float* gates, int* offsets, int* sorted_token, float* sorted_gate,
-                          int* inv, int M, int E, int k, hipStream_t s) {
+                          int* inv, int M, int E, int k, int extra_group, hipStream_t s) {
   if (M <= 0) return 0;
-  if (E < 1 || E > 4096) return JLE_BAD_ARG;
-  return launch_align(ids, gates, offsets, sorted_token, sorted_gate, inv, M, E, k, s);
+  if (E < 1 || E > 4096 || k < 1 || M % k) return JLE_BAD_ARG;
+  return launch_align(ids, gates, offsets, sorted_token, sorted_gate, inv, M, E, k, extra_group ? M / k : 0, s);
 }

@@ -27,8 +27,8 @@ _SIGNATURES = {
     "jle_qk_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_paged_attention_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _vp],
     "jle_moe_route": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
-    "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
-    "jle_moe_route_align": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "jle_moe_route_align": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
@@ -36,7 +36,7 @@ _SIGNATURES = {
     "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i,
                              _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
-    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -210,12 +210,18 @@ class HipOps:
     SKINNY_DENSE_ROWS = 16  # the fused gate|up projection of a dense feed-forward: beyond this the BLAS library
 
     def gemm_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
-                    variant=0, tiled=False):
+                    variant=0, tiled=False, b_last=None, tiled_last=False):
         """bfloat16 weight-streaming product on MFMA for few rows (see ``gemm_skinny.hip``); with ``swiglu`` the
-        result is ``silu(gate) * up`` of the two halves of ``b``'s rows."""
+        result is ``silu(gate) * up`` of the two halves of ``b``'s rows.  ``b_last``: one more group behind
+        ``b``'s, its matrix a tensor of its own (``offsets`` then has an entry more)."""
         if b.dim() == 2:
             b = b.unsqueeze(0)
         g, nout, k = b.shape
+        if b_last is not None:
+            self._chk(b_last, torch.bfloat16, (nout, k), "the last group's matrix")
+            if offsets is None or offsets.numel() != g + 2:
+                raise KernelError("a last group with a matrix of its own needs offsets for one group more")
+            g += 1
         m = rows if rows is not None else (a_rows.numel() if a_rows is not None else a.shape[0])
         self._chk(a, torch.bfloat16, None, "A")
         self._chk(b, torch.bfloat16, None, "B")
@@ -226,7 +232,7 @@ class HipOps:
         out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
                           device=a.device)
         self._call("jle_gemm_skinny", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
-                   int(out_f32), m, nout, k, g, m, variant, int(tiled))
+                   int(out_f32), m, nout, k, g, m, variant, int(tiled), _p(b_last), int(tiled_last))
         return out
 
     def gemm_grouped(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
@@ -443,41 +449,63 @@ class HipOps:
         gates = torch.empty(n, top_k, dtype=torch.float32, device=dev)
         logits = torch.empty(n, e, dtype=torch.float32, device=dev)
         if group:
+            # (with one more group behind the experts' that holds every token once: a shared expert's rows)
             m = n * top_k
-            offsets = torch.empty(e + 1, dtype=torch.int32, device=dev)
-            sorted_token = torch.empty(m, dtype=torch.int32, device=dev)
-            sorted_gate = torch.empty(m, dtype=torch.float32, device=dev)
+            offsets = torch.empty(e + 2, dtype=torch.int32, device=dev)
+            sorted_token = torch.empty(m + n, dtype=torch.int32, device=dev)
+            sorted_gate = torch.empty(m + n, dtype=torch.float32, device=dev)
             inv = torch.empty(m, dtype=torch.int32, device=dev)
             self._call("jle_moe_route_align", _p(h32), _p(router), _p(ids), _p(gates), _p(logits), _p(offsets),
-                       _p(sorted_token), _p(sorted_gate), _p(inv), n, d, e, top_k)
+                       _p(sorted_token), _p(sorted_gate), _p(inv), n, d, e, top_k, 1)
             grouping = (offsets, sorted_token, sorted_gate, inv)
             return (ids, gates, logits, grouping) if want_logits else (ids, gates, grouping)
         self._call("jle_moe_route", _p(h32), _p(router), _p(ids), _p(gates), _p(logits), n, d, e, top_k)
         return (ids, gates, logits) if want_logits else (ids, gates)
 
-    def moe_align(self, expert_ids, gates, num_experts: int):
+    def moe_align(self, expert_ids, gates, num_experts: int, extra_group: bool = False):
+        """Stable grouping of the (token, choice) pairs by expert: offsets ``[E + 1]``, the token and the gate of
+        every sorted row, and where each pair went.  ``extra_group``: one more group behind the experts' that
+        holds every token once, in order, with gate 1 (the rows of a shared expert)."""
         n, k = expert_ids.shape
         m = n * k
+        x = n if extra_group else 0
         dev = expert_ids.device
         self._chk(expert_ids, torch.int32, None, "expert ids")
         self._chk(gates, torch.float32, (n, k), "gates")
-        offsets = torch.empty(num_experts + 1, dtype=torch.int32, device=dev)
-        sorted_token = torch.empty(m, dtype=torch.int32, device=dev)
-        sorted_gate = torch.empty(m, dtype=torch.float32, device=dev)
+        offsets = torch.empty(num_experts + (2 if extra_group else 1), dtype=torch.int32, device=dev)
+        sorted_token = torch.empty(m + x, dtype=torch.int32, device=dev)
+        sorted_gate = torch.empty(m + x, dtype=torch.float32, device=dev)
         inv = torch.empty(m, dtype=torch.int32, device=dev)
         self._call("jle_moe_align", _p(expert_ids), _p(gates), _p(offsets), _p(sorted_token), _p(sorted_gate), _p(inv),
-                   m, num_experts, k)
+                   m, num_experts, k, int(extra_group))
         return offsets, sorted_token, sorted_gate, inv
 
-    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None):
+    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None,
+                    shared_weights=None):
+        """``shared``: a shared expert's output, or ``shared_weights``: its (gate|up, down) matrices, row-major."""
         n, d = h.shape
         e, f2, _ = w_gate_up.shape
         k = expert_ids.shape[1]
-        if grouping is None:
-            grouping = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e)
-        offsets, sorted_token, sorted_gate, inv = grouping
+        m = n * k
         mfma = h.dtype == torch.bfloat16 and d % 8 == 0 and (f2 // 2) % 8 == 0
-        if mfma and n * k <= 2 * self.SKINNY_MAX_ROWS:  # few rows: the cost is streaming the chosen experts' weights
+        # a step of few tokens streams the shared expert's gate|up matrix in the launch of the routed experts', as
+        # one more group (the cost of such a step is the kernels' getting started, not their work); its down
+        # matrix stays with the library: row-major with rows 2^n bytes apart, it streams badly through this kernel
+        fuse = (shared is None and shared_weights is not None and mfma and n <= self.SKINNY_DENSE_ROWS
+                and m <= 2 * self.SKINNY_MAX_ROWS and tuple(shared_weights[0].shape) == (f2, d))
+        if grouping is None or (fuse and grouping[0].numel() != e + 2):
+            grouping = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e, extra_group=fuse)
+        offsets, sorted_token, sorted_gate, inv = grouping
+        if fuse:
+            act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,
+                                   tiled=tiled, b_last=shared_weights[0], rows=m + n)
+            routed = self.gemm_skinny(act, w_down, offsets=offsets[: e + 1], tiled=tiled, rows=m)
+            return ExpertSum(routed, inv, k, self.linear(act[m:], shared_weights[1]), n, d)
+        if shared is None and shared_weights is not None:
+            shared = self.linear(self.swiglu_linear(h, shared_weights[0]), shared_weights[1])
+        if grouping[0].numel() != e + 1:  # (made with the extra group: the kernels below do not know of it)
+            offsets, sorted_token, sorted_gate = offsets[: e + 1], sorted_token[:m], sorted_gate[:m]
+        if mfma and m <= 2 * self.SKINNY_MAX_ROWS:  # few rows: the cost is streaming the chosen experts' weights
             act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,
                                    tiled=tiled)
             routed = self.gemm_skinny(act, w_down, offsets=offsets, tiled=tiled)

@@ -167,12 +167,15 @@ class ReferenceOps:
         ids, gates = order.to(torch.int32), torch.sigmoid(vals)
         return (ids, gates, None) if group else (ids, gates)
 
-    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None):
+    def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None,
+                    shared_weights=None):
         """``sum_j  W_down[e_j] (silu(g_j W_gate[e_j] h) * (g_j W_up[e_j] h))`` per token,
         plus ``shared`` if given; float32 result.  ``w_gate_up`` is ``[E, 2F, D]`` (gate rows then
         up rows), ``w_down`` ``[E, D, F]``.  Activations between the two products are
         rounded to the run dtype, as the kernels store them."""
         assert not tiled, "the plain ops read row-major weights"
+        if shared is None and shared_weights is not None:
+            shared = self.linear(self.swiglu_linear(h, shared_weights[0]), shared_weights[1])
         n, d = h.shape
         f = w_down.shape[2]
         out = torch.zeros(n, d, dtype=torch.float32, device=h.device)

@@ -78,8 +78,6 @@ class MoESigmoidShared(FeedForward):
         if forced is not None:
             expert_ids, gates = forced
             grouping = None
-        shared = None
-        if self.shared_inter:
-            shared = ops.linear(ops.swiglu_linear(h, self.params["shared_gate_up"]), self.params["shared_down"])
-        return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"], shared,
-                               tiled=self.tiled, grouping=grouping)
+        shared = (self.params["shared_gate_up"], self.params["shared_down"]) if self.shared_inter else None
+        return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"],
+                               shared_weights=shared, tiled=self.tiled, grouping=grouping)

@@ -278,9 +278,9 @@ def test_router_and_grouping_in_one_call(ops, n, d, e, k):
     kernels.  Either way the same as route, then align."""
     h, w = _rand(n, d, seed=1), _rand(e, d, scale=0.05, seed=2)
     ids, gates, logits = ops.moe_route(h, w, k, want_logits=True)
-    want = ops.moe_align(ids, gates, e)
     ids2, gates2, logits2, grouping = ops.moe_route(h, w, k, want_logits=True, group=True)
     assert torch.equal(ids, ids2) and torch.equal(gates, gates2) and torch.equal(logits, logits2)
+    want = ops.moe_align(ids, gates, e, extra_group=True)
     for a, b in zip(want, grouping):
         assert torch.equal(a, b)
 
@@ -324,6 +324,37 @@ def test_moe_experts(ops, ref, dt, n, d, f, e, k):
     assert torch.equal(ops.gather_rows(lazy, idx), got[idx.long()])
 
 
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("n,d,f,e,k", [(1, 64, 32, 4, 1), (9, 96, 48, 3, 2), (16, 256, 64, 16, 1), (17, 64, 32, 4, 1),
+                                       (50, 96, 48, 5, 1)])
+def test_moe_experts_with_the_shared_expert_given_by_its_matrices(ops, ref, dt, tiled, n, d, f, e, k):
+    """Up to 16 tokens the shared expert's gate|up product goes through the routed experts' launch as one more
+    group (its matrix stays row-major beside experts in either layout); beyond, through the library.  The same sum."""
+    from jax_llm_examples_amd.ops.layout import can_tile, tile_
+
+    h = _rand(n, d, dt=dt, seed=1)
+    wgu, wd = _rand(e, 2 * f, d, dt=dt, scale=0.2, seed=2), _rand(e, d, f, dt=dt, scale=0.2, seed=3)
+    sgu, sd = _rand(2 * f, d, dt=dt, scale=0.2, seed=4), _rand(d, f, dt=dt, scale=0.2, seed=5)
+    g = torch.Generator().manual_seed(5)
+    ids = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(n)]).to(torch.int32).to(DEV)
+    gates = torch.rand(n, k, generator=g).to(DEV)
+    want = ref.moe_experts(h, ids, gates, wgu, wd, shared_weights=(sgu, sd))
+    if tiled:
+        if dt != torch.bfloat16 or not (can_tile(wgu) and can_tile(wd)):
+            pytest.skip("the streaming layout is for bfloat16 matrices of whole tiles")
+        wgu, wd = wgu.clone(), wd.clone()
+        tile_(wgu)
+        tile_(wd)
+    lazy = ops.moe_experts(h, ids, gates, wgu, wd, shared_weights=(sgu, sd), tiled=tiled)
+    _assert_close_to_scale(ops.materialize(lazy), want, dt)
+    # with the grouping that the router's own call makes (an extra group always), and with one made without
+    for extra in (True, False):
+        grouping = ops.moe_align(ids, gates, e, extra_group=extra)
+        lazy = ops.moe_experts(h, ids, gates, wgu, wd, shared_weights=(sgu, sd), tiled=tiled, grouping=grouping)
+        _assert_close_to_scale(ops.materialize(lazy), want, dt)
+
+
 def test_moe_align_is_a_stable_grouping(ops):
     g = torch.Generator().manual_seed(0)
     ids = torch.randint(0, 7, (300, 2), generator=g).to(torch.int32).to(DEV)
@@ -338,6 +369,11 @@ def test_moe_align_is_a_stable_grouping(ops):
         assert torch.equal(inv[rows], torch.arange(int(off[e]), int(off[e + 1]), dtype=torch.int32))  # in order
         assert torch.equal(tok[off[e]: off[e + 1]], (rows // 2).to(torch.int32))
     assert torch.equal(gate[inv.long()], gates.flatten().cpu())
+    # one more group that holds every token once
+    off2, tok2, gate2, inv2 = (t.cpu() for t in ops.moe_align(ids, gates, 7, extra_group=True))
+    assert torch.equal(off2[:8], off) and off2[8] == 900 and torch.equal(inv2, inv)
+    assert torch.equal(tok2[:600], tok) and torch.equal(tok2[600:], torch.arange(300, dtype=torch.int32))
+    assert torch.equal(gate2[:600], gate) and torch.equal(gate2[600:], torch.ones(300))
 
 
 @pytest.mark.parametrize("dt", DT)
