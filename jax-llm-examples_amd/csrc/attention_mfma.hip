@@ -33,6 +33,7 @@ using namespace jle;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;  // (register arrays of HIP's uint4 may end up in scratch)
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -188,7 +189,14 @@ __device__ __forceinline__ void common_range(const Columns (&col)[CT], int& lo, 
 }
 
 // The shared core.  DH: head size; CT: column tiles.  Returns through m, l, acc (O^T, unnormalised).
-template <int DH, int CT>
+// ONCE: the keys and values are read by this wavefront alone in this launch (decode): loads that the caches need
+// not keep, which stream faster.
+template <bool ONCE, typename V>
+__device__ __forceinline__ V load_kv(const void* p) {
+  return ONCE ? __builtin_nontemporal_load(reinterpret_cast<const V*>(p)) : *reinterpret_cast<const V*>(p);
+}
+
+template <int DH, int CT, bool ONCE>
 __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv,
                                        const int* __restrict__ table, const Columns (&col)[CT], int k_lo, int k_hi,
                                        int hk, int Hq, int Hkv, int ps, float scale_log2, float (&m)[CT],
@@ -256,10 +264,10 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
         const bf16_t* krow = kbase + (size_t)(offs[tt] + c16) * DH + g * 8;
         const bf16_t* vcol = kbase + (size_t)Hkv * plane + offs[tt] + 4 * g;  // + d * ps
 #pragma unroll
-        for (int c = 0; c < KC; ++c) kraw[tt][c] = *reinterpret_cast<const u32x4*>(krow + c * 32);
+        for (int c = 0; c < KC; ++c) kraw[tt][c] = load_kv<ONCE, u32x4>(krow + c * 32);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          const uint2 t = *reinterpret_cast<const uint2*>(vcol + (size_t)(dt * 16 + c16) * ps);
+          const u32x2 t = load_kv<ONCE, u32x2>(vcol + (size_t)(dt * 16 + c16) * ps);
           if (tt == 0) {
             vnext[dt].x = t.x;
             vnext[dt].y = t.y;
@@ -351,7 +359,7 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention
   float m[CT], l[CT];
   f32x4 acc[CT][DH / 16];
   bool bad = false;
-  attend<DH, CT>(q, kv, block_table + (size_t)token_segment[n0] * table_width, col, k_lo, k_hi, hk, Hq, Hkv, ps,
+  attend<DH, CT, false>(q, kv, block_table + (size_t)token_segment[n0] * table_width, col, k_lo, k_hi, hk, Hq, Hkv, ps,
                  scale_log2, m, l, acc, bad);
   bad = __any(bad);
 #pragma unroll
@@ -642,7 +650,7 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention
   float m[CT], l[CT];
   f32x4 acc[CT][DH / 16];
   bool bad = false;
-  attend<DH, CT>(q, kv, block_table + (size_t)token_segment[n] * table_width, col, k_lo, k_hi, hk, Hq, Hkv, ps,
+  attend<DH, CT, true>(q, kv, block_table + (size_t)token_segment[n] * table_width, col, k_lo, k_hi, hk, Hq, Hkv, ps,
                  scale_log2, m, l, acc, bad);
   bad = __any(bad);
 #pragma unroll

@@ -97,8 +97,9 @@ __device__ __forceinline__ void stream_block(const bf16_t* __restrict__ X, const
   auto ask_weights = [&](u32x4 (&w)[2][2], int s) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      w[ks][0] = *reinterpret_cast<const u32x4*>(w0 + (size_t)(2 * s + ks) * 512);
-      w[ks][1] = *reinterpret_cast<const u32x4*>(w1 + (size_t)(2 * s + ks) * 512);
+      // (read by this wavefront alone, once: loads that the caches need not keep, which stream faster)
+      w[ks][0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w0 + (size_t)(2 * s + ks) * 512));
+      w[ks][1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w1 + (size_t)(2 * s + ks) * 512));
     }
   };
   auto put = [&](const u32x4 (&x)[CPT], bf16_t* buf) {
