@@ -6,15 +6,17 @@
 // The cost is reading W once; the rows of X are few (up to 16 * MT per group and block).  The
 // weights are the MFMA's A operand (16 weight rows x 32 k per instruction, each lane reads 16
 // contiguous bytes of a weight row), the activations its B operand (16 tokens), so no data is
-// transposed.  A block is 4 wavefronts that split K between them (k-blocks of 32 interleaved, so
-// together they read 256 contiguous bytes of each weight row) and add their partial sums in
-// shared memory in a fixed order.  Each block owns two 16-row weight tiles (SWIGLU: the gate tile
+// transposed.  A block is 4 wavefronts that split K between them (pairs of k-blocks of 32, interleaved)
+// and add their partial sums in shared memory in a fixed order.  Each block owns two 16-row weight tiles (SWIGLU: the gate tile
 // and its up tile, so the activation is formed in the epilogue); grid = (row tiles, token tiles,
 // groups); blocks of groups without rows leave at once.
 //
-// W is either row-major or in the streaming layout (`tiled`): tiles of 16 rows x 32 k stored as the
-// kilobyte one A-operand load reads (lane g * 16 + r: row r, elements 8 g ..), tiles along K
-// contiguous - then every load instruction of a wavefront reads one contiguous kilobyte.
+// W is either in the streaming layout (`tiled`): tiles of 16 rows x 32 k stored as the kilobyte one
+// A-operand load reads (lane g * 16 + r: row r, elements 8 g ..), tiles along K contiguous - then
+// every load instruction of a wavefront reads one contiguous kilobyte; or row-major: then a load
+// instruction reads whole 128-byte lines of 8 rows, and the lines are turned into A operands through
+// shared memory.  Either way the weights are read with loads that the caches need not keep (measured
+// on MI355X: a stream of such loads reads 7.2 TB/s, of plain ones 6.4).
 #include "common.h"
 
 using namespace jle;
@@ -26,10 +28,8 @@ __device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
   const uint4 v = *reinterpret_cast<const uint4*>(p);
   return __builtin_bit_cast(bf16x8, v);
 }
-// weights are read once per step: a load that the caches need not keep (measured on MI355X: a stream of such
-// loads reads 7.2 TB/s, of plain ones 6.4)
 typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
-__device__ __forceinline__ bf16x8 load8_once(const bf16_t* p) {
+__device__ __forceinline__ bf16x8 load_once(const bf16_t* p) {
   const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
   return __builtin_bit_cast(bf16x8, v);
 }
@@ -54,6 +54,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
                                                           int tiled_last) {
   static_assert(RT == 2 || !SWIGLU, "the fused activation needs the gate tile and the up tile");
   __shared__ float red[WAVES][RT * MT * 4][64];
+  __shared__ __attribute__((aligned(16))) bf16_t turn[WAVES][RT * 16 * 72];  // (row-major weights only)
   const int e = blockIdx.z;
   int row_lo = 0, row_hi = M;
   if (offsets != nullptr) {
@@ -71,29 +72,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
   }
   const int half = Nout >> 1;
   const int base = SWIGLU ? blockIdx.x * 16 : blockIdx.x * (16 * RT);  // first output column of the block
-  int ra0, ra1;  // the weight rows this lane reads
-  if (SWIGLU) {
-    ra0 = min(base + r, half - 1);
-    ra1 = half + ra0;
-  } else {
-    ra0 = min(base + r, Nout - 1);
-    ra1 = min(base + 16 + r, Nout - 1);
-  }
   const int nkb = (K + 31) >> 5;
-  const bf16_t* a0;
-  const bf16_t* a1;
-  int kb_stride;  // elements from one k-block of 32 to the next
+  const bf16_t* a0 = We;
+  const bf16_t* a1 = We;
   if (tiled) {  // rows and K are whole tiles
     const int ntile = Nout >> 4;
     const int t0 = SWIGLU ? (base >> 4) : min(base >> 4, ntile - 1);
     const int t1 = SWIGLU ? ((half + base) >> 4) : min((base >> 4) + 1, ntile - 1);
     a0 = We + (size_t)t0 * nkb * 512 + lane * 8;
     a1 = We + (size_t)t1 * nkb * 512 + lane * 8;
-    kb_stride = 512;
-  } else {
-    a0 = We + (size_t)ra0 * K + g * 8;
-    a1 = We + (size_t)ra1 * K + g * 8;
-    kb_stride = 32;
   }
   const bf16_t* xb[MT];
   bool xv[MT];
@@ -110,23 +97,94 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
     acc0[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     acc1[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  for (int kb0 = wave; kb0 < nkb; kb0 += WAVES * kUnroll) {
-    bf16x8 A0[kUnroll], A1[kUnroll], B[kUnroll][MT];
+  if (tiled) {
+    // streaming layout: a load instruction reads a contiguous kilobyte that nobody else wants, straight into
+    // the A operand
+    // (a wavefront takes every WAVES-th pair of k-blocks, as with row-major weights below: the same sums in the
+    // same order, so the layout does not change a single bit of the result)
+    static_assert(kUnroll % 2 == 0, "k-blocks are taken in pairs");
+    for (int L0 = wave; 2 * L0 < nkb; L0 += WAVES * (kUnroll / 2)) {
+      bf16x8 A0[kUnroll], A1[kUnroll], B[kUnroll][MT];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int kb = kb0 + WAVES * u;
-      const bool ok = kb < nkb && (kb * 32 + g * 8) < K;  // K is a multiple of 8
-      A0[u] = ok ? load8_once(a0 + (size_t)kb * kb_stride) : zero8();
-      if (RT == 2) A1[u] = ok ? load8_once(a1 + (size_t)kb * kb_stride) : zero8();
+      for (int u = 0; u < kUnroll; ++u) {
+        const int kb = 2 * (L0 + WAVES * (u >> 1)) + (u & 1);
+        const bool ok = kb < nkb;  // (K is whole k-blocks in this layout)
+        A0[u] = ok ? load_once(a0 + (size_t)kb * 512) : zero8();
+        if (RT == 2) A1[u] = ok ? load_once(a1 + (size_t)kb * 512) : zero8();
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) B[u][mt] = (ok && xv[mt]) ? load8(xb[mt] + kb * 32) : zero8();
+        for (int mt = 0; mt < MT; ++mt) B[u][mt] = (ok && xv[mt]) ? load8(xb[mt] + kb * 32) : zero8();
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          acc0[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A0[u], B[u][mt], acc0[mt], 0, 0, 0);
+          if (RT == 2) acc1[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[u], B[u][mt], acc1[mt], 0, 0, 0);
+        }
+      }
     }
+  } else {
+    // row-major: a load instruction reads whole 128-byte lines, 8 lanes a row's line (64 k), 8 rows; the A
+    // operand wants 16 rows x 32 k with 4 lanes a row, so the lines go through a piece of shared memory of the
+    // wavefront's own (rows 144 bytes apart: neither writing nor reading collides).  A wavefront takes every
+    // WAVES-th line.
+    constexpr int UL = kUnroll / 2;  // lines on their way
+    constexpr int LROW = 72;                             // elements from row to row in shared memory
+    bf16_t* buf = turn[wave];
+    const int lr = lane >> 3, lc = lane & 7;
+    const bf16_t* src[RT][2];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        acc0[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A0[u], B[u][mt], acc0[mt], 0, 0, 0);
-        if (RT == 2) acc1[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1[u], B[u][mt], acc1[mt], 0, 0, 0);
+      for (int h = 0; h < 2; ++h) {
+        const int rr = h * 8 + lr;
+        int row;
+        if (SWIGLU) row = min(base + rr, half - 1) + (t == 1 ? half : 0);
+        else row = min(base + 16 * t + rr, Nout - 1);
+        src[t][h] = We + (size_t)row * K + lc * 8;
+      }
+    const int nlines = (K + 63) >> 6;
+    for (int L0 = wave; L0 < nlines; L0 += WAVES * UL) {
+      u32x4 raw[UL][RT][2];
+      bf16x8 B[UL][2][MT];
+#pragma unroll
+      for (int u = 0; u < UL; ++u) {
+        const int L = L0 + WAVES * u;
+        const bool ok = L < nlines && (L * 64 + lc * 8) < K;  // K is a multiple of 8
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            raw[u][t][h] = ok ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src[t][h] + (size_t)L * 64))
+                              : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const int kb = 2 * L + ks;
+          const bool okb = L < nlines && (kb * 32 + g * 8) < K;
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) B[u][ks][mt] = (okb && xv[mt]) ? load8(xb[mt] + kb * 32) : zero8();
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UL; ++u) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            *reinterpret_cast<u32x4*>(buf + (t * 16 + h * 8 + lr) * LROW + lc * 8) = raw[u][t][h];
+        // (one wavefront's accesses to shared memory are carried out in their order: no barrier)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const bf16x8 A0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(buf + r * LROW + (g + 4 * ks) * 8));
+          bf16x8 A1 = A0;
+          if (RT == 2)
+            A1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(buf + (16 + r) * LROW + (g + 4 * ks) * 8));
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            acc0[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A0, B[u][ks][mt], acc0[mt], 0, 0, 0);
+            if (RT == 2) acc1[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(A1, B[u][ks][mt], acc1[mt], 0, 0, 0);
+          }
+        }
       }
     }
   }
