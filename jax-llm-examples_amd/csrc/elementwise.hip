@@ -100,6 +100,20 @@ __device__ __forceinline__ f32x4_t load4<bf16_t>(const bf16_t* p) {
   return f32x4_t{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
                  __uint_as_float(r.y & 0xffff0000u)};
 }
+// the same for data that this launch reads once and the caches need not keep
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+template <typename T>
+__device__ __forceinline__ f32x4_t load4_once(const T* p);
+template <>
+__device__ __forceinline__ f32x4_t load4_once<float>(const float* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
+}
+template <>
+__device__ __forceinline__ f32x4_t load4_once<bf16_t>(const bf16_t* p) {
+  const u32x2_t r = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
+  return f32x4_t{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
+                 __uint_as_float(r.y & 0xffff0000u)};
+}
 template <typename T>
 __device__ __forceinline__ void store4(T* p, f32x4_t v);
 template <>
@@ -114,10 +128,10 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v) {
 template <typename DT>
 __device__ __forceinline__ f32x4_t delta_at4(const Delta<DT>& delta, size_t n, int d, int D) {
   f32x4_t v = {0.f, 0.f, 0.f, 0.f};
-  if (delta.plain != nullptr) v = load4<DT>(delta.plain + n * D + d);
+  if (delta.plain != nullptr) v = load4_once<DT>(delta.plain + n * D + d);
   if (delta.routed != nullptr) {
-    for (int j = 0; j < delta.k; ++j) v += load4<DT>(delta.routed + (size_t)delta.inv[n * delta.k + j] * D + d);
-    if (delta.shared != nullptr) v += load4<DT>(delta.shared + n * D + d);
+    for (int j = 0; j < delta.k; ++j) v += load4_once<DT>(delta.routed + (size_t)delta.inv[n * delta.k + j] * D + d);
+    if (delta.shared != nullptr) v += load4_once<DT>(delta.shared + n * D + d);
   }
   return v;
 }
@@ -147,10 +161,10 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
     const int d = (threadIdx.x + THREADS * i) * 4;
     v[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     if (d < D) {
-      v[i] = load4<float>(x + base + d);
+      v[i] = load4_once<float>(x + base + d);
       if (add) {
         v[i] += delta_at4<DT>(delta, n, d, D);
-        store4<float>(x + base + d, v[i]);
+        __builtin_nontemporal_store(v[i], reinterpret_cast<f32x4_t*>(x + base + d));
       }
       ss += v[i][0] * v[i][0];
       ss += v[i][1] * v[i][1];

@@ -91,17 +91,22 @@ class HipOps:
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise KernelError("the HIP kernels need a GPU")
         self.lib = load_library()
+        self._fn = {name: getattr(self.lib, name) for name in _SIGNATURES}
+        self._device_index = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        self._raw_stream = raw if raw is not None else (lambda i: torch.cuda.current_stream(i).cuda_stream)
         # true float32 products: no reduced-precision matrix mode
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
         torch.set_float32_matmul_precision("highest")
 
     # ------------------------------------------------------------------ helpers
-    def _stream(self):
-        return torch.cuda.current_stream(self.device).cuda_stream
+    def _stream(self) -> int:
+        """The current stream's handle (a decode step asks hundreds of times: the raw query, not a Stream object)."""
+        return self._raw_stream(self._device_index)
 
     def _call(self, name: str, *args) -> None:
-        rc = getattr(self.lib, name)(*args, self._stream())
+        rc = self._fn[name](*args, self._stream())
         if rc != 0:
             if rc < 0:
                 raise KernelError(f"{name}: the kernel refuses these sizes or options")
@@ -181,7 +186,14 @@ class HipOps:
 
     # ------------------------------------------------------------------ matrix products
     def linear(self, h, w, out_dtype=None):
-        """``h @ w.T`` through the BLAS library (float32: true float32)."""
+        """``h @ w.T``: through the BLAS library (float32: true float32); a few bfloat16 rows through the
+        weight-streaming kernel, which is as fast there and much cheaper to launch (measured on 7168 x 5120 and
+        5120 x 5120; not where the rows of ``w`` lie a multiple of 4 KB apart, which that kernel streams badly)."""
+        if (h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_LINEAR_ROWS and w.dim() == 2
+                and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and (w.shape[1] * 2) % 4096
+                and h.is_contiguous() and w.is_contiguous()):
+            out = self.gemm_skinny(h, w)
+            return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
         out = torch.matmul(h, w.t())
         return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
 
@@ -208,6 +220,7 @@ class HipOps:
 
     SKINNY_MAX_ROWS = 64  # up to here a product is a stream of the weights: the MFMA weight-streaming kernel
     SKINNY_DENSE_ROWS = 16  # the fused gate|up projection of a dense feed-forward: beyond this the BLAS library
+    SKINNY_LINEAR_ROWS = 8  # plain projections (q|k|v, o, down)
 
     def gemm_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
                     variant=0, tiled=False, b_last=None, tiled_last=False):
