@@ -187,11 +187,9 @@ class HipOps:
     # ------------------------------------------------------------------ matrix products
     def linear(self, h, w, out_dtype=None):
         """``h @ w.T``: through the BLAS library (float32: true float32); a few bfloat16 rows through the
-        weight-streaming kernel, which is as fast there and much cheaper to launch (measured on 7168 x 5120 and
-        5120 x 5120; not where the rows of ``w`` lie a multiple of 4 KB apart, which that kernel streams badly)."""
+        weight-streaming kernel, which is as fast there or faster and much cheaper to launch."""
         if (h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_LINEAR_ROWS and w.dim() == 2
-                and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and (w.shape[1] * 2) % 4096
-                and h.is_contiguous() and w.is_contiguous()):
+                and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and h.is_contiguous() and w.is_contiguous()):
             out = self.gemm_skinny(h, w)
             return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
         out = torch.matmul(h, w.t())
@@ -501,19 +499,19 @@ class HipOps:
         k = expert_ids.shape[1]
         m = n * k
         mfma = h.dtype == torch.bfloat16 and d % 8 == 0 and (f2 // 2) % 8 == 0
-        # a step of few tokens streams the shared expert's gate|up matrix in the launch of the routed experts', as
-        # one more group (the cost of such a step is the kernels' getting started, not their work); its down
-        # matrix stays with the library: row-major with rows 2^n bytes apart, it streams badly through this kernel
+        # a step of few tokens streams the shared expert's matrices in the launches of the routed experts', as one
+        # more group: the cost of such a step is the kernels' getting started, not their work
         fuse = (shared is None and shared_weights is not None and mfma and n <= self.SKINNY_DENSE_ROWS
-                and m <= 2 * self.SKINNY_MAX_ROWS and tuple(shared_weights[0].shape) == (f2, d))
+                and m <= 2 * self.SKINNY_MAX_ROWS and tuple(shared_weights[0].shape) == (f2, d)
+                and tuple(shared_weights[1].shape) == (d, f2 // 2))
         if grouping is None or (fuse and grouping[0].numel() != e + 2):
             grouping = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e, extra_group=fuse)
         offsets, sorted_token, sorted_gate, inv = grouping
         if fuse:
             act = self.gemm_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate, swiglu=True,
                                    tiled=tiled, b_last=shared_weights[0], rows=m + n)
-            routed = self.gemm_skinny(act, w_down, offsets=offsets[: e + 1], tiled=tiled, rows=m)
-            return ExpertSum(routed, inv, k, self.linear(act[m:], shared_weights[1]), n, d)
+            both = self.gemm_skinny(act, w_down, offsets=offsets, tiled=tiled, b_last=shared_weights[1])
+            return ExpertSum(both[:m], inv, k, both[m:], n, d)
         if shared is None and shared_weights is not None:
             shared = self.linear(self.swiglu_linear(h, shared_weights[0]), shared_weights[1])
         if grouping[0].numel() != e + 1:  # (made with the extra group: the kernels below do not know of it)

@@ -329,8 +329,8 @@ def test_moe_experts(ops, ref, dt, n, d, f, e, k):
 @pytest.mark.parametrize("n,d,f,e,k", [(1, 64, 32, 4, 1), (9, 96, 48, 3, 2), (16, 256, 64, 16, 1), (17, 64, 32, 4, 1),
                                        (50, 96, 48, 5, 1)])
 def test_moe_experts_with_the_shared_expert_given_by_its_matrices(ops, ref, dt, tiled, n, d, f, e, k):
-    """Up to 16 tokens the shared expert's gate|up product goes through the routed experts' launch as one more
-    group (its matrix stays row-major beside experts in either layout); beyond, through the library.  The same sum."""
+    """Up to 16 tokens the shared expert's products go through the routed experts' launches as one more group
+    (its matrices stay row-major beside experts in either layout); beyond, through the library.  The same sum."""
     from jax_llm_examples_amd.ops.layout import can_tile, tile_
 
     h = _rand(n, d, dt=dt, seed=1)
