@@ -125,20 +125,29 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v) {
   *reinterpret_cast<uint2*>(p) = uint2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
 }
 
-template <typename DT>
+// STREAM: the step is so large that what this launch reads and writes will have left the caches before anyone
+// wants it again (loads and stores that the caches need not keep); a step of few tokens is better off finding the
+// residual in the cache half a layer later.
+template <bool STREAM, typename T>
+__device__ __forceinline__ f32x4_t load4_as(const T* p) {
+  return STREAM ? load4_once<T>(p) : load4<T>(p);
+}
+
+template <bool STREAM, typename DT>
 __device__ __forceinline__ f32x4_t delta_at4(const Delta<DT>& delta, size_t n, int d, int D) {
   f32x4_t v = {0.f, 0.f, 0.f, 0.f};
-  if (delta.plain != nullptr) v = load4_once<DT>(delta.plain + n * D + d);
+  if (delta.plain != nullptr) v = load4_as<STREAM, DT>(delta.plain + n * D + d);
   if (delta.routed != nullptr) {
-    for (int j = 0; j < delta.k; ++j) v += load4_once<DT>(delta.routed + (size_t)delta.inv[n * delta.k + j] * D + d);
-    if (delta.shared != nullptr) v += load4_once<DT>(delta.shared + n * D + d);
+    for (int j = 0; j < delta.k; ++j)
+      v += load4_as<STREAM, DT>(delta.routed + (size_t)delta.inv[n * delta.k + j] * D + d);
+    if (delta.shared != nullptr) v += load4_as<STREAM, DT>(delta.shared + n * D + d);
   }
   return v;
 }
 
 // Rows whose width is a multiple of 8 (and 16-byte aligned arrays): a thread takes CPT pieces of 4
 // neighbouring elements, piece = thread, thread + THREADS, ...; up to THREADS * CPT * 4 wide.
-template <typename DT, typename OT, int THREADS, int CPT>
+template <typename DT, typename OT, int THREADS, int CPT, bool STREAM>
 __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ x, Delta<DT> delta,
                                                                   const float* __restrict__ w, float eps,
                                                                   OT* __restrict__ out, float* __restrict__ out32,
@@ -161,10 +170,11 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
     const int d = (threadIdx.x + THREADS * i) * 4;
     v[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     if (d < D) {
-      v[i] = load4_once<float>(x + base + d);
+      v[i] = load4_as<STREAM, float>(x + base + d);
       if (add) {
-        v[i] += delta_at4<DT>(delta, n, d, D);
-        __builtin_nontemporal_store(v[i], reinterpret_cast<f32x4_t*>(x + base + d));
+        v[i] += delta_at4<STREAM, DT>(delta, n, d, D);
+        if (STREAM) __builtin_nontemporal_store(v[i], reinterpret_cast<f32x4_t*>(x + base + d));
+        else store4<float>(x + base + d, v[i]);
       }
       ss += v[i][0] * v[i][0];
       ss += v[i][1] * v[i][1];
@@ -221,9 +231,15 @@ static void launch_add_rmsnorm(float* x, Delta<DT> delta, const float* w, float 
   // (which kernel: by the width and the arrays' alignment only, so a row's result is the same in any batch)
   const uintptr_t all = (uintptr_t)x | (uintptr_t)delta.plain | (uintptr_t)delta.routed | (uintptr_t)delta.shared |
                         (uintptr_t)w | (uintptr_t)out | (uintptr_t)out32;
-  if (D % 8 == 0 && (all & 15) == 0 && D > 1024 && D <= 8192)  // (rows of any of the arrays then start 16-byte aligned)
-    hipLaunchKernelGGL((add_rmsnorm_vec_kernel<DT, OT, 256, 8>), g, dim3(256), 0, s, x, delta, w, eps, (OT*)out, out32,
-                       D);
+  if (D % 8 == 0 && (all & 15) == 0 && D > 1024 && D <= 8192) {  // (rows of any of the arrays then start 16-byte aligned)
+    // (the same arithmetic either way: only where the data are kept differs)
+    if ((size_t)N * D >= ((size_t)4 << 20))
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<DT, OT, 256, 8, true>), g, dim3(256), 0, s, x, delta, w, eps,
+                         (OT*)out, out32, D);
+    else
+      hipLaunchKernelGGL((add_rmsnorm_vec_kernel<DT, OT, 256, 8, false>), g, dim3(256), 0, s, x, delta, w, eps,
+                         (OT*)out, out32, D);
+  }
   else if (D <= 1024)
     hipLaunchKernelGGL((add_rmsnorm_reg_kernel<DT, OT, 256, 4>), g, dim3(256), 0, s, x, delta, w, eps, (OT*)out, out32,
                        D);
