@@ -4,31 +4,32 @@
 //   Y[t, f] = silu(s * gate) * (s * up),  gate/up = rows f and F + f of W[g(t)]   (SWIGLU, s = scale[t])
 //
 // The cost is reading W once; the rows of X are few (up to 16 * MT per group and block).  The
-// weights are the MFMA's A operand (16 weight rows x 32 k per instruction, each lane reads 16
-// contiguous bytes of a weight row), the activations its B operand (16 tokens), so no data is
-// transposed.  A block is 4 wavefronts that split K between them (pairs of k-blocks of 32, interleaved)
-// and add their partial sums in shared memory in a fixed order.  Each block owns two 16-row weight tiles (SWIGLU: the gate tile
+// weights are the MFMA's A operand (16 weight rows x 32 k per instruction), the activations its B
+// operand (16 tokens).  A block is WAVES wavefronts that split K between them (pairs of k-blocks of
+// 32, interleaved; every block starts at another pair and wraps round) and add their partial sums in
+// shared memory in a fixed order.  A block owns one or two 16-row weight tiles (SWIGLU: the gate tile
 // and its up tile, so the activation is formed in the epilogue); grid = (row tiles, token tiles,
 // groups); blocks of groups without rows leave at once.
 //
 // W is either in the streaming layout (`tiled`): tiles of 16 rows x 32 k stored as the kilobyte one
 // A-operand load reads (lane g * 16 + r: row r, elements 8 g ..), tiles along K contiguous - then
-// every load instruction of a wavefront reads one contiguous kilobyte; or row-major: then a load
-// instruction reads whole 128-byte lines of 8 rows, and the lines are turned into A operands through
-// shared memory.  Either way the weights are read with loads that the caches need not keep (measured
-// on MI355X: a stream of such loads reads 7.2 TB/s, of plain ones 6.4).
+// every load instruction of a wavefront reads one contiguous kilobyte, straight into the operand; or
+// row-major: then a load instruction reads whole 128-byte lines of 8 rows, and the lines are turned
+// into A operands through shared memory.  Either way the weights are read with loads that the caches
+// need not keep (measured on MI355X: a stream of such loads reads 7.2 TB/s, of plain ones 6.4), and
+// the sums are formed in the same order, so the layout does not change a bit of the result.
 #include "common.h"
 
 using namespace jle;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) {
   const uint4 v = *reinterpret_cast<const uint4*>(p);
   return __builtin_bit_cast(bf16x8, v);
 }
-typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 __device__ __forceinline__ bf16x8 load_once(const bf16_t* p) {
   const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
   return __builtin_bit_cast(bf16x8, v);
