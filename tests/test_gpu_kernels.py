@@ -438,7 +438,7 @@ def test_sampling_frequencies_follow_softmax(ops):
 
 
 @pytest.mark.parametrize("m,nout,k", [(1, 64, 64), (8, 70, 104), (16, 33, 32), (17, 96, 40), (40, 500, 264),
-                                       (64, 130, 5120)])
+                                       (64, 130, 5120), (5, 1000, 8192), (3, 80, 1096)])
 @pytest.mark.parametrize("out_f32", [False, True])
 def test_weight_streaming_product(ops, ref, m, nout, k, out_f32):
     a, b = _rand(m, k, dt=torch.bfloat16, seed=1), _rand(nout, k, dt=torch.bfloat16, scale=0.1, seed=2)
