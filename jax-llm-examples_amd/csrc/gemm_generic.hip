@@ -13,7 +13,29 @@ using namespace jle;
 
 constexpr int BM = 64, BN = 64, BK = 16, PAD = 4;
 
-template <typename T, typename OT>
+// four consecutive k of a row, as float32 (VEC: one load; K is a multiple of 4 and the arrays are 16-byte aligned)
+template <bool VEC, typename T>
+__device__ __forceinline__ void load_k4(const T* p, int k, int K, bool ok, float (&v)[4]) {
+  if (VEC) {
+    if (ok && k < K) {
+      if constexpr (sizeof(T) == 4) {
+        const float4 r = *reinterpret_cast<const float4*>(p + k);
+        v[0] = r.x, v[1] = r.y, v[2] = r.z, v[3] = r.w;
+      } else {
+        const uint2 r = *reinterpret_cast<const uint2*>(p + k);
+        v[0] = __uint_as_float(r.x << 16), v[1] = __uint_as_float(r.x & 0xffff0000u);
+        v[2] = __uint_as_float(r.y << 16), v[3] = __uint_as_float(r.y & 0xffff0000u);
+      }
+    } else {
+      v[0] = v[1] = v[2] = v[3] = 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (ok && k + i < K) ? Num<T>::load(p + k + i) : 0.f;
+  }
+}
+
+template <typename T, typename OT, bool VEC>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B,
                                                            OT* __restrict__ C, const int* __restrict__ offsets,
                                                            const int* __restrict__ a_rows,
@@ -60,11 +82,13 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
     for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
 
   for (int k0 = 0; k0 < K; k0 += BK) {
+    float av[4], bv[4];
+    load_k4<VEC, T>(a_ptr, k0 + lk, K, a_ok, av);
+    load_k4<VEC, T>(b_ptr, k0 + lk, K, b_ok, bv);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int k = k0 + lk + i;
-      As[lk + i][lr] = (a_ok && k < K) ? Num<T>::load(a_ptr + k) : 0.f;
-      Bs[lk + i][lr] = (b_ok && k < K) ? Num<T>::load(b_ptr + k) : 0.f;
+      As[lk + i][lr] = av[i];
+      Bs[lk + i][lr] = bv[i];
     }
     __syncthreads();
 #pragma unroll
@@ -103,9 +127,17 @@ JLE_API int jle_gemm_generic(const void* A, const void* B, void* C, const int* o
   const int row_tiles = (M + BM - 1) / BM + (offsets != nullptr ? G : 0);
   if (row_tiles > 65535) return JLE_BAD_ARG;
   dim3 g((Nout + BN - 1) / BN, row_tiles), b(256);
-#define LAUNCH(T, OT)                                                                                          \
-  hipLaunchKernelGGL((gemm_generic_kernel<T, OT>), g, b, 0, s, (const T*)A, (const T*)B, (OT*)C, offsets, a_rows, \
-                     scale, M, Nout, K, G)
+  // (the same sums in the same order either way)
+  const bool vec = K % 4 == 0 && (((uintptr_t)A | (uintptr_t)B) & 15) == 0;
+#define LAUNCH(T, OT)                                                                                             \
+  do {                                                                                                            \
+    if (vec)                                                                                                      \
+      hipLaunchKernelGGL((gemm_generic_kernel<T, OT, true>), g, b, 0, s, (const T*)A, (const T*)B, (OT*)C, offsets, \
+                         a_rows, scale, M, Nout, K, G);                                                           \
+    else                                                                                                          \
+      hipLaunchKernelGGL((gemm_generic_kernel<T, OT, false>), g, b, 0, s, (const T*)A, (const T*)B, (OT*)C,        \
+                         offsets, a_rows, scale, M, Nout, K, G);                                                  \
+  } while (0)
   if (in_bf16) {
     if (out_f32) LAUNCH(bf16_t, float); else LAUNCH(bf16_t, bf16_t);
   } else {

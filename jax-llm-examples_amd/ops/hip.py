@@ -25,7 +25,8 @@ _SIGNATURES = {
     "jle_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
     "jle_moe_combine": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_qk_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _vp],
-    "jle_paged_attention_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_paged_attention_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
+                                    _vp, _vp],
     "jle_moe_route": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_moe_route_align": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
@@ -338,6 +339,7 @@ class HipOps:
         return q
 
     PREFILL_TILE = 32  # tokens per prefill work item (the kernels take 16 or 32)
+    GENERIC_SPLIT_BELOW = 2048  # the float32-arithmetic attention: fewer (token, head) pairs than this share their keys
     DECODE_ITEMS = 1024  # decode attention: work items (wavefronts) that run at once, one per SIMD
     DECODE_MIN_SPLIT = 128  # keys per work item at least (fewer: the merge costs more than the spreading gains)
     DECODE_FIT_SPLIT = 1024  # ... at most, to make the items fit in one go
@@ -440,9 +442,24 @@ class HipOps:
             raise KernelError(f"attention kernels: head size {dh} is not supported (a multiple of 8, at most 256)")
         if hq % hk:
             raise KernelError(f"attention kernels: {hq} query heads are no multiple of {hk} kv heads")
+        # few tokens with many keys (decode): each query's keys are shared between several wavefronts
+        splits, tiles_per_split, ws_ml, ws_o = 1, 0, None, None
+        waves = n * hq
+        if waves < self.GENERIC_SPLIT_BELOW:
+            if meta is not None:
+                longest = max(s0 + ln for s0, ln in zip(meta.seg_starts, meta.seg_lens))
+            else:
+                longest = int(positions.max()) + 1
+            tiles = -(-longest // 64)
+            want = min(tiles, -(-self.GENERIC_SPLIT_BELOW // waves))
+            if want > 1:
+                tiles_per_split = -(-tiles // want)
+                splits = -(-tiles // tiles_per_split)
+                ws_ml = torch.empty(waves * splits * 2, dtype=torch.float32, device=q.device)
+                ws_o = torch.empty(waves * splits * dh, dtype=torch.float32, device=q.device)
         self._call("jle_paged_attention_generic", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
                    _p(block_table), block_table.shape[1], mode, param, float(scale), self._is_bf16(q), n, hq, hk, dh,
-                   ps)
+                   ps, splits, tiles_per_split, _p(ws_ml), _p(ws_o))
         return out
 
     # ------------------------------------------------------------------ routed experts
