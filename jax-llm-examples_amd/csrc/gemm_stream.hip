@@ -29,7 +29,6 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 namespace {
 
 constexpr int kRows = 192;       // rows of a pass
-constexpr int NT = kRows / 16;   // B tiles of a pass
 constexpr int BK = 64;           // k per stage (two MFMA steps)
 constexpr int XAHEAD = 2;        // stages between asking for rows and using them (two register sets, two buffers)
 constexpr int WAHEAD = 4;        // the same for weights (four register sets)
