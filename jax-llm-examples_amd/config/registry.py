@@ -64,9 +64,11 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_name(top: Mapping[str, Any]) -> str:
     archs = top.get("architectures")
-    if not archs:
-        raise UnknownArchitectureError("config.json has no 'architectures' entry")
-    return str(archs[0])
+    if archs:
+        return str(archs[0])
+    if top.get("model_type"):  # (a folder written without the entry)
+        return str(top["model_type"])
+    raise UnknownArchitectureError("config.json has neither an 'architectures' entry nor a 'model_type'")
 
 
 def read_config_json(model_dir: str | os.PathLike) -> dict:

@@ -20,7 +20,8 @@ from ..weights.bindings import TensorBinding
 
 
 class Llama4Architecture:
-    names = ("Llama4ForConditionalGeneration", "Llama4ForCausalLM")
+    # config.json's "architectures" entries, and its "model_type" values for folders that carry only those
+    names = ("Llama4ForConditionalGeneration", "Llama4ForCausalLM", "llama4", "llama4_text")
     optional_prefixes = ("language_model.",)
     ignored_prefixes = ("vision_model.", "multi_modal_projector.")
 

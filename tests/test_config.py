@@ -31,6 +31,17 @@ def test_parse_and_round_trip(name, tmp_path):
     assert arch2 is arch and cfg2 == cfg
 
 
+def test_model_type_stands_in_for_a_missing_architectures_entry():
+    from jax_llm_examples_amd.config.registry import architecture_name
+    from tiny_configs import tiny_config_json
+
+    top = {k: v for k, v in tiny_config_json("A").items() if k != "architectures"}
+    top["model_type"] = "llama4_text"
+    assert get_architecture(architecture_name(top)) is get_architecture("Llama4ForCausalLM")
+    with pytest.raises(UnknownArchitectureError, match="neither"):
+        architecture_name({"hidden_size": 8})
+
+
 def test_text_config_is_used_when_present():
     top = tiny_config_json("B")
     assert "text_config" in top
