@@ -4,7 +4,8 @@ The reference converts checkpoints in two stages with per-tensor asserts
 (``llama4/llama4_jax/chkpt_utils.py:80-159``) and raises on unknown, unexpected,
 duplicate and missing names (``chkpt_utils.py:159, 257-261, 274-275``).  Here
 the checkpoint is read directly; every problem found (missing tensors,
-unexpected tensors, wrong shapes) is reported in one :class:`WeightsError`.
+unexpected tensors, tensors met twice, wrong shapes) is reported in one
+:class:`WeightsError`.
 """
 from __future__ import annotations
 
@@ -20,15 +21,19 @@ from .safetensors_io import SafetensorsFile
 
 
 class WeightsError(ValueError):
-    def __init__(self, missing, unexpected, wrong_shape, where: str) -> None:
+    def __init__(self, missing, unexpected, wrong_shape, where: str, duplicate=()) -> None:
         self.missing = list(missing)
         self.unexpected = list(unexpected)
         self.wrong_shape = list(wrong_shape)
+        self.duplicate = list(duplicate)  # (name, where it was met first, where again)
         lines = [f"weights in {where} do not match the model:"]
         if self.missing:
             lines.append(f"  missing ({len(self.missing)}): " + ", ".join(self.missing))
         if self.unexpected:
             lines.append(f"  unexpected ({len(self.unexpected)}): " + ", ".join(self.unexpected))
+        if self.duplicate:
+            lines.append(f"  met twice ({len(self.duplicate)}): " + ", ".join(
+                f"{n} ({a} and {b})" for n, a, b in self.duplicate))
         if self.wrong_shape:
             lines.append(f"  wrong shape ({len(self.wrong_shape)}): " + ", ".join(
                 f"{n} is {list(got)}, expected {list(exp)}" for n, got, exp in self.wrong_shape))
@@ -66,12 +71,20 @@ def load_weights(model, model_dir: str, bindings: list[TensorBinding], *, option
     files = [SafetensorsFile(p) for p in _checkpoint_files(os.fspath(model_dir))]
     try:
         found: dict[str, tuple[SafetensorsFile, str]] = {}
-        unexpected = []
+        duplicate = []
         for f in files:
             for raw in f.names():
                 if any(raw.startswith(p) for p in ignored_prefixes):
                     continue
-                found[_canonical(raw, optional_prefixes)] = (f, raw)
+                name = _canonical(raw, optional_prefixes)
+                if name in found:
+                    # in two files, or once with and once without an optional prefix: which one is meant cannot
+                    # be known (the reference refuses a parameter that is set twice, chkpt_utils.py:261)
+                    f0, raw0 = found[name]
+                    duplicate.append((name, f"{raw0} in {os.path.basename(f0.path)}",
+                                      f"{raw} in {os.path.basename(f.path)}"))
+                    continue
+                found[name] = (f, raw)
         expected = {b.name: b for b in bindings}
         missing = [n for n in expected if n not in found]
         unexpected = [n for n in found if n not in expected]
@@ -81,8 +94,8 @@ def load_weights(model, model_dir: str, bindings: list[TensorBinding], *, option
                 f, raw = found[n]
                 if f.shape(raw) != tuple(b.shape):
                     wrong.append((n, f.shape(raw), tuple(b.shape)))
-        if missing or unexpected or wrong:
-            raise WeightsError(missing, unexpected, wrong, os.fspath(model_dir))
+        if missing or unexpected or wrong or duplicate:
+            raise WeightsError(missing, unexpected, wrong, os.fspath(model_dir), duplicate)
         params = model.named_parameters()
         for n, b in expected.items():
             f, raw = found[n]

@@ -116,3 +116,46 @@ def test_sharded_checkpoint_with_index(model_dirs, tmp_path):
     a = load_model(str(tmp_path / "sh"), "float32", "cpu").named_parameters()
     b = load_model(model_dirs["A"], "float32", "cpu").named_parameters()
     assert all(torch.equal(a[k], b[k]) for k in b)
+
+
+def _folder_with(tmp_path, name, files, index=None):
+    d = tmp_path / name
+    os.makedirs(d)
+    for fn, tensors in files.items():
+        save_file(tensors, str(d / fn))
+    if index is not None:
+        with open(d / "model.safetensors.index.json", "w") as f:
+            json.dump({"weight_map": index}, f)
+    with open(d / "config.json", "w") as f:
+        json.dump(tiny_config_json("A"), f)
+    return str(d)
+
+
+def test_a_tensor_in_two_shards_is_an_error_not_the_last_one_read(model_dirs, tmp_path):
+    raw = load_file(os.path.join(model_dirs["A"], "model.safetensors"))
+    names = sorted(raw)
+    half = len(names) // 2
+    twice = "model.layers.1.self_attn.o_proj.weight"
+    first = {k: raw[k] for k in names[:half]}
+    second = {k: raw[k] for k in names[half:]}
+    first[twice] = raw[twice]
+    second[twice] = torch.zeros_like(raw[twice])  # a stale copy: loading it silently would give wrong weights
+    d = _folder_with(tmp_path, "dup", {"model-00001-of-00002.safetensors": first,
+                                       "model-00002-of-00002.safetensors": second})
+    with pytest.raises(WeightsError) as ei:
+        load_model(d, "float32", "cpu")
+    e = ei.value
+    assert [n for n, _, _ in e.duplicate] == [twice]
+    assert not e.missing and not e.unexpected and not e.wrong_shape
+    assert "met twice (1)" in str(e) and "model-00001-of-00002.safetensors" in str(e) \
+        and "model-00002-of-00002.safetensors" in str(e)
+
+
+def test_a_tensor_with_and_without_the_optional_prefix_is_an_error(model_dirs, tmp_path):
+    raw = load_file(os.path.join(model_dirs["A"], "model.safetensors"))
+    raw["language_model.model.norm.weight"] = raw["model.norm.weight"] * 2
+    d = _folder_with(tmp_path, "dup2", {"model.safetensors": raw})
+    with pytest.raises(WeightsError) as ei:
+        load_model(d, "float32", "cpu")
+    assert [n for n, _, _ in ei.value.duplicate] == ["model.norm.weight"]
+    assert "language_model.model.norm.weight" in str(ei.value)
