@@ -4,6 +4,9 @@
 //                     (0 = all).  The noise of a token depends only on (seed, counter, token id),
 //                     so a request's choice does not depend on what else is in the batch.
 #include "common.h"
+#include "jle.h"
+
+#include <mutex>
 
 using namespace jle;
 
@@ -189,4 +192,49 @@ JLE_API int jle_sample(const float* logits, const float* temperature, const int*
     JLE_LAUNCH_CHECK();
   }
   return 0;
+}
+
+// ------------------------------------------------------------------ the same without a workspace argument
+// The blocks' choices of the two-stage kernels go into an array that is part of the loaded code object, so the
+// call allocates nothing (see jle.h).  Every GPU that runs this library holds its own copy of the array, at an
+// address of its own, until the process ends.
+constexpr int kStaticSampleEntries = JLE_SAMPLE_STATIC_MAX_ENTRIES;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[(size_t)kStaticSampleEntries * (sizeof(float) + sizeof(int))];
+
+// The array's address on each device, asked for once per device (in host code the array's name is only a handle
+// for this query, never an address that a kernel could use).
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+static int scratch_on_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return JLE_BAD_ARG;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+JLE_API int jle_sample_static(const float* logits, const float* temperature, const int* top_k, const int* seeds,
+                              const int* counters, int* out, int M, int V, int any_top_k, hipStream_t s) {
+  if (M <= 0) return 0;
+  if (V <= 0 || M > 65535) return JLE_BAD_ARG;
+  const long long S = ((long long)V + kChunk - 1) / kChunk;
+  if ((long long)M * S > kStaticSampleEntries) return JLE_BAD_ARG;  // more (row, chunk) pairs than the array holds
+  void* base = nullptr;
+  if (int rc = scratch_on_current_device(&base)) return rc;
+  // Every (row, chunk) entry that the second stage reads is written by the first stage of this same call, so
+  // what an earlier call left in the array is never seen and nothing has to be cleared.
+  float* part_v = reinterpret_cast<float*>(base);
+  int* part_i = reinterpret_cast<int*>(static_cast<unsigned char*>(base) + (size_t)kStaticSampleEntries * sizeof(float));
+  return jle_sample(logits, temperature, top_k, seeds, counters, out, part_v, part_i, M, V, any_top_k, s);
 }
