@@ -48,8 +48,7 @@ def main() -> int:
     from jax_llm_examples_amd.config.presets import PRESETS, preset
     from jax_llm_examples_amd.config.registry import architecture_name, get_architecture
     from jax_llm_examples_amd.engine import ModelRunner, StepEntry, get_ops, random_model
-    from jax_llm_examples_amd.engine.accounting import decode_step_bytes, prefill_flops
-    from jax_llm_examples_amd.parts.feed_forward import MoESigmoidShared
+    from jax_llm_examples_amd.engine.accounting import StepWatcher, decode_step_bytes, prefill_flops
     from jax_llm_examples_amd.sampling import Sampler, SamplingParams
 
     dev = "cuda:0"
@@ -113,9 +112,9 @@ def main() -> int:
         last = torch.randint(0, V, (batch,), generator=gen).tolist()
         params, ctr = [greedy] * batch, [0] * batch
 
-        def one(record=False):
+        def one(tap=None):
             nonlocal last
-            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(ids, last)], record_routing=record)
+            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(ids, last)], tap=tap)
             last = sampler(logits, params, ctr)
 
         for _ in range(warmup):
@@ -126,14 +125,12 @@ def main() -> int:
             one()
         torch.cuda.synchronize()
         sec = (time.perf_counter() - t1) / steps
-        distinct = {}
-        one(record=True)
-        for li, b in enumerate(model.blocks):
-            ff = b.feed_forward
-            if isinstance(ff, MoESigmoidShared) and ff.last_routing is not None:
-                distinct[li] = int(torch.unique(ff.last_routing[0]).numel())
+        watcher = StepWatcher()  # one more step, watched: which experts its tokens choose
+        one(tap=watcher)
+        distinct = {li: int(torch.unique(seen["routing"][0]).numel()) for li, b in enumerate(model.blocks)
+                    for seen in [watcher.seen.get(id(b.feed_forward))] if seen and "routing" in seen}
         contexts = [cache.num_tokens(r) for r in ids]
-        nbytes = decode_step_bytes(model, cache, contexts, distinct)
+        nbytes = decode_step_bytes(model, cache, contexts, watcher)
         for rid in ids:
             runner.finish(rid)
         print(f"[bench] decode batch {batch}: {sec * 1e3:.2f} ms/step, {batch / sec:.1f} tok/s, "

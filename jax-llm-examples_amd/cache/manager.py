@@ -10,8 +10,13 @@ overwritten.  Here pages are given back when a request ends and as soon as a
 group's retention rule (chunk or window) has passed them.
 
 Runs of the model's order with the same ``(kv heads, head size, retention)``
-form a *group*: they share page ids and one block table per request, and each
-has a tensor ``[num_pages, 2, kv_heads, page_size, head_dim]`` of its own.
+(and the same further per-token tensors, if any) form a *group*: they share page
+ids and one block table per request, and each has a tensor ``[num_pages, 2,
+kv_heads, page_size, head_dim]`` of its own (and ``[num_pages, page_size,
+*shape]`` for every further per-token tensor it declares).  Every group has a
+pool of its own size: a group whose retention rule lets go of old tokens never
+holds more than a chunk (or window) plus one step's portion per request, so it
+needs far fewer pages than a group that keeps everything (:func:`pool_sizes`).
 """
 from __future__ import annotations
 
@@ -27,15 +32,27 @@ from .pages import OutOfPages, OutOfSlots, PagePool, SlotPool
 @dataclasses.dataclass
 class CacheGroup:
     index: int
-    kv_heads: int
+    kv_heads: int  # 0: no keys and values in the attention kernels' layout
     head_dim: int
     retention: tuple
     cache_ids: list[int]
     pool: PagePool
-    tensors: dict[int, torch.Tensor]
+    tensors: dict[int, torch.Tensor]  # per run: [pages, 2, kv_heads, page_size, head_dim]
+    paged: tuple = ()  # further per-token tensors: (name, shape) pairs
+    pages: dict[int, dict[str, torch.Tensor]] = dataclasses.field(default_factory=dict)  # per run, by name
+    itemsize: int = 2
 
-    def bytes_per_token(self, itemsize: int) -> int:
-        return len(self.cache_ids) * 2 * self.kv_heads * self.head_dim * itemsize
+    def bytes_per_token(self, itemsize: int | None = None) -> int:
+        """Bytes one token takes in this group, over all its runs."""
+        if itemsize is None:
+            itemsize = self.itemsize
+        per_run = 2 * self.kv_heads * self.head_dim
+        for _, shape in self.paged:
+            n = 1
+            for d in shape:
+                n *= d
+            per_run += n
+        return len(self.cache_ids) * per_run * itemsize
 
 
 @dataclasses.dataclass
@@ -58,6 +75,96 @@ class CacheView:
     state: Optional[torch.Tensor] = None
     attn_meta: Optional[object] = None
     group: Optional[int] = None
+    pages: Optional[dict] = None  # further per-token tensors of this run, by name: [pages, page_size, *shape]
+
+
+def group_key(need: CacheNeed):
+    """Runs whose needs give the same key share page ids and block tables; ``None``: no pages."""
+    if need.kv is None and not need.paged:
+        return None
+    kv = (0, 0) if need.kv is None else (int(need.kv[0]), int(need.kv[1]))
+    paged = tuple((str(n), tuple(int(d) for d in shape)) for n, shape in need.paged)
+    return (kv, paged, tuple(need.retention))
+
+
+def plan_groups(needs: dict[int, CacheNeed]) -> list[tuple[tuple, list[int]]]:
+    """The groups the manager will form, in its order: ``(key, cache ids)``."""
+    out: list[tuple[tuple, list[int]]] = []
+    index: dict[tuple, int] = {}
+    for cid in sorted(needs):
+        key = group_key(needs[cid])
+        if key is None:
+            continue
+        if key not in index:
+            index[key] = len(out)
+            out.append((key, []))
+        out[index[key]][1].append(cid)
+    return out
+
+
+def tokens_held_at_most(retention: tuple, max_step_tokens: int, max_seq_len: Optional[int]) -> Optional[int]:
+    """The most tokens of one request that a group with this retention rule holds at any time
+    (``None``: no bound but the sequence's length): what the rule keeps for the next query plus the
+    portion of the running step, whose pages are given back only after it."""
+    kind = retention[0]
+    cap = None
+    if kind in ("chunk", "window"):
+        cap = int(retention[1]) + max_step_tokens
+    if max_seq_len is not None:
+        cap = max_seq_len if cap is None else min(cap, max_seq_len)
+    return cap
+
+
+def pool_sizes(needs: dict[int, CacheNeed], *, page_size: int, itemsize: int, max_requests: int,
+               max_step_tokens: int, max_seq_len: Optional[int] = None, cache_tokens: Optional[int] = None,
+               memory_bytes: Optional[int] = None) -> dict[int, int]:
+    """Pages for every group's pool.  Either ``cache_tokens`` (the tokens that a group which keeps
+    everything can hold) or ``memory_bytes`` (what all pools together may take: then the largest
+    such number of tokens that fits).  A group that lets go of old tokens gets at most what
+    ``max_requests`` requests can hold of it (whole pages, and one more per request for a portion
+    that does not start at a page's edge)."""
+    groups = plan_groups(needs)
+    caps, page_bytes = [], []
+    for (kv, paged, retention), cids in groups:
+        held = tokens_held_at_most(retention, max_step_tokens, max_seq_len)
+        caps.append(None if held is None else max_requests * (-(-held // page_size) + 1))
+        per = 2 * kv[0] * kv[1]
+        for _, shape in paged:
+            n = 1
+            for d in shape:
+                n *= d
+            per += n
+        page_bytes.append(len(cids) * per * page_size * itemsize)
+
+    def sizes(pages_unbounded: int) -> list[int]:
+        return [pages_unbounded if c is None else min(c, pages_unbounded) for c in caps]
+
+    if cache_tokens is not None:
+        want = -(-cache_tokens // page_size)
+    elif memory_bytes is not None:
+        def total(p):
+            return sum(b * n for b, n in zip(page_bytes, sizes(p)))
+
+        lo, hi = 0, 1
+        while total(hi) <= memory_bytes and hi < (1 << 40):
+            if all(c is not None and c <= hi for c in caps):
+                break  # every pool is at its bound: more pages would hold nothing
+            lo, hi = hi, hi * 2
+        if total(hi) <= memory_bytes:
+            lo = hi
+        while lo + 1 < hi:
+            mid = (lo + hi) // 2
+            if total(mid) <= memory_bytes:
+                lo = mid
+            else:
+                hi = mid
+        want = lo
+        if want < 1:
+            raise ValueError(f"{memory_bytes} bytes do not hold one page of every group "
+                             f"({sum(page_bytes)} bytes)")
+    else:
+        raise ValueError("give cache_tokens or memory_bytes")
+    return dict(enumerate(sizes(want)))
 
 
 class CacheManager:
@@ -84,19 +191,17 @@ class CacheManager:
         self.group_of: dict[int, int] = {}
         self.state: dict[int, torch.Tensor] = {}
         self.requests: dict[object, RequestEntry] = {}
-        by_key: dict[tuple, CacheGroup] = {}
+        item = torch.empty((), dtype=dtype).element_size()
+        for key, cids in plan_groups(needs):
+            (hk, dh), paged, retention = key
+            i = len(self.groups)
+            n = num_pages[i] if isinstance(num_pages, dict) else num_pages
+            g = CacheGroup(i, hk, dh, retention, list(cids), PagePool(n), {}, paged=paged, itemsize=item)
+            self.groups.append(g)
+            for cid in cids:
+                self.group_of[cid] = i
         for cid in sorted(needs):
             need = needs[cid]
-            if need.kv is not None:
-                key = (need.kv[0], need.kv[1], tuple(need.retention))
-                g = by_key.get(key)
-                if g is None:
-                    n = num_pages[len(self.groups)] if isinstance(num_pages, dict) else num_pages
-                    g = CacheGroup(len(self.groups), need.kv[0], need.kv[1], tuple(need.retention), [], PagePool(n), {})
-                    by_key[key] = g
-                    self.groups.append(g)
-                g.cache_ids.append(cid)
-                self.group_of[cid] = g.index
             if need.state_shape is not None:
                 self.state[cid] = torch.zeros(
                     (max_requests, *need.state_shape), dtype=need.state_dtype or torch.float32, device=self.device
@@ -104,9 +209,14 @@ class CacheManager:
         fill = float("nan") if poison else 0.0
         for g in self.groups:
             for cid in g.cache_ids:
-                g.tensors[cid] = torch.full(
-                    (g.pool.num_pages, 2, g.kv_heads, page_size, g.head_dim), fill, dtype=dtype, device=self.device
-                )
+                if g.kv_heads:
+                    g.tensors[cid] = torch.full(
+                        (g.pool.num_pages, 2, g.kv_heads, page_size, g.head_dim), fill, dtype=dtype, device=self.device
+                    )
+                g.pages[cid] = {
+                    name: torch.full((g.pool.num_pages, page_size, *shape), fill, dtype=dtype, device=self.device)
+                    for name, shape in g.paged
+                }
 
     # ------------------------------------------------------------------ requests
     def add_request(self, rid) -> RequestEntry:
@@ -209,6 +319,9 @@ class CacheManager:
             idx = torch.tensor(pages, dtype=torch.long, device=self.device)
             for t in g.tensors.values():
                 t.index_fill_(0, idx, float("nan"))
+            for named in g.pages.values():
+                for t in named.values():
+                    t.index_fill_(0, idx, float("nan"))
 
     # ------------------------------------------------------------------ queries
     def num_tokens(self, rid) -> int:
@@ -241,8 +354,12 @@ class CacheManager:
                 )
 
     def bytes_per_token(self) -> int:
-        item = torch.empty((), dtype=self.dtype).element_size()
-        return sum(g.bytes_per_token(item) for g in self.groups)
+        return sum(g.bytes_per_token() for g in self.groups)
+
+    def pool_bytes(self) -> int:
+        """Device memory of all page pools."""
+        return sum(g.bytes_per_token() * self.page_size * g.pool.num_pages for g in self.groups)
 
 
-__all__ = ["CacheManager", "CacheView", "CacheGroup", "OutOfPages", "OutOfSlots"]
+__all__ = ["CacheManager", "CacheView", "CacheGroup", "OutOfPages", "OutOfSlots", "pool_sizes", "plan_groups",
+           "tokens_held_at_most"]

@@ -20,6 +20,12 @@ from typing import Any, Mapping, Optional
 from .specs import LayerSpec, ModelPlan, default_order, part
 
 
+def _number(v):
+    """A whole number stays an integer (checkpoints store ``floor_scale`` as one)."""
+    f = float(v)
+    return int(f) if f.is_integer() else f
+
+
 class ConfigError(ValueError):
     """A config.json that cannot describe a model: names the key at fault."""
 
@@ -70,7 +76,7 @@ class Llama4TextConfig:
     rope_theta: float
     rope_scaling: Optional[RopeScaling]
     attn_temperature_tuning: bool
-    floor_scale: float
+    floor_scale: float  # (held as an integer where config.json has a whole number, and written back so)
     attn_scale: float
     tie_word_embeddings: bool = False
     torch_dtype: str = "bfloat16"
@@ -150,7 +156,7 @@ class Llama4TextConfig:
             rope_theta=float(d["rope_theta"]),
             rope_scaling=rope_scaling,
             attn_temperature_tuning=bool(d.get("attn_temperature_tuning", False)),
-            floor_scale=float(d.get("floor_scale", 8192)),
+            floor_scale=_number(d.get("floor_scale", 8192)),
             attn_scale=float(d.get("attn_scale", 0.1)),
             tie_word_embeddings=bool(d.get("tie_word_embeddings", top.get("tie_word_embeddings", False))),
             torch_dtype=str(d.get("torch_dtype", top.get("torch_dtype", "bfloat16"))),

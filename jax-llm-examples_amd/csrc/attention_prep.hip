@@ -1,6 +1,7 @@
-// After the fused q|k|v projection: rotary embedding over adjacent pairs, weightless
-// L2 (rms) norm of q and k, position-dependent query scale, and the write of k and v
-// into their page.  One wavefront per (token, head); everything in float32.
+// After the fused q|k|v projection: rotary embedding (adjacent or half-split pairs, over the whole head
+// or its leading part), rms norm of q and k over the head (with or without weights, before or after the
+// rotation), position-dependent query scale, and the write of k and v into their page.  One wavefront per
+// (token, head); everything in float32.
 //
 // Page layout, per page and kv head: keys [page_size][head_dim] (a key's elements contiguous),
 // values [head_dim][page_size] (one element of all the page's tokens contiguous), so that both
@@ -11,11 +12,16 @@ using namespace jle;
 
 constexpr int kMaxPairsPerLane = 4;  // head_dim <= 512
 
+// pairing 0: pairs (x[2j], x[2j+1]); 1: pairs (x[j], x[j + rotary_dim / 2]).  Elements from rotary_dim on are not
+// rotated.  norm_wq / norm_wk: weights of the norm (null: none).  norm_first: the norm (statistics from the
+// unrotated head) and its weights come before the rotation.
 template <typename T>
 __global__ void qk_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ kv_cache,
                                   const int* __restrict__ positions, const int* __restrict__ slot_mapping,
                                   const float* __restrict__ inv_freq, float norm_eps, float floor_scale,
-                                  float attn_scale, int Hq, int Hkv, int dh, int page_size, int write_kv) {
+                                  float attn_scale, int Hq, int Hkv, int dh, int page_size, int write_kv, int pairing,
+                                  int rotary_dim, const float* __restrict__ norm_wq,
+                                  const float* __restrict__ norm_wk, int norm_first) {
   const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const bool is_q = h < Hq;
   const bool is_v = h >= Hq + Hkv;
@@ -23,30 +29,59 @@ __global__ void qk_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
   const T* src = qkv + ((size_t)n * (Hq + 2 * Hkv) + h) * dh;
   const int pos = positions[n];
   const int half = dh >> 1;
+  const int rh = inv_freq != nullptr ? rotary_dim >> 1 : 0;  // rotated pairs
+  const bool normed = !is_v && norm_eps >= 0.f;
+  const float* nw = is_q ? norm_wq : norm_wk;
   float a[kMaxPairsPerLane], b[kMaxPairsPerLane];
+  int e1[kMaxPairsPerLane], e2[kMaxPairsPerLane];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < kMaxPairsPerLane; ++i) {
     const int j = lane + 64 * i;
     a[i] = 0.f;
     b[i] = 0.f;
+    e1[i] = 0;
+    e2[i] = 0;
     if (j < half) {
-      float x1 = Num<T>::load(src + 2 * j), x2 = Num<T>::load(src + 2 * j + 1);
-      if (!is_v && inv_freq != nullptr) {
+      if (pairing == 0 || j >= rh) {
+        e1[i] = pairing == 0 ? 2 * j : 2 * rh + 2 * (j - rh);
+        e2[i] = e1[i] + 1;
+      } else {
+        e1[i] = j;
+        e2[i] = j + rh;
+      }
+      a[i] = Num<T>::load(src + e1[i]);
+      b[i] = Num<T>::load(src + e2[i]);
+      ss += a[i] * a[i] + b[i] * b[i];
+    }
+  }
+  if (normed && norm_first) {
+    const float m0 = 1.0f / sqrtf(wave_sum(ss) / (float)dh + norm_eps);
+#pragma unroll
+    for (int i = 0; i < kMaxPairsPerLane; ++i) {
+      a[i] *= m0 * (nw != nullptr ? nw[e1[i]] : 1.f);
+      b[i] *= m0 * (nw != nullptr ? nw[e2[i]] : 1.f);
+    }
+  }
+  ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMaxPairsPerLane; ++i) {
+    const int j = lane + 64 * i;
+    if (j < half) {
+      if (!is_v && j < rh) {
         const float ang = (float)pos * inv_freq[j];
         const float sn = sinf(ang), cs = cosf(ang);
-        const float r1 = x1 * cs - x2 * sn;
-        const float r2 = x2 * cs + x1 * sn;
-        x1 = r1;
-        x2 = r2;
+        const float r1 = a[i] * cs - b[i] * sn;
+        const float r2 = b[i] * cs + a[i] * sn;
+        a[i] = r1;
+        b[i] = r2;
       }
-      a[i] = x1;
-      b[i] = x2;
-      ss += x1 * x1 + x2 * x2;
+      ss += a[i] * a[i] + b[i] * b[i];
     }
   }
   float mul = 1.f;
-  if (!is_v && norm_eps >= 0.f) {
+  const bool norm_after = normed && !norm_first;
+  if (norm_after) {
     const float tot = wave_sum(ss);
     mul = 1.0f / sqrtf(tot / (float)dh + norm_eps);
   }
@@ -73,8 +108,10 @@ __global__ void qk_prepare_kernel(const T* __restrict__ qkv, T* __restrict__ q_o
   for (int i = 0; i < kMaxPairsPerLane; ++i) {
     const int j = lane + 64 * i;
     if (j < half) {
-      Num<T>::store(dst + (size_t)(2 * j) * stride, a[i] * mul);
-      Num<T>::store(dst + (size_t)(2 * j + 1) * stride, b[i] * mul);
+      const float w1 = (norm_after && nw != nullptr) ? nw[e1[i]] : 1.f;
+      const float w2 = (norm_after && nw != nullptr) ? nw[e2[i]] : 1.f;
+      Num<T>::store(dst + (size_t)e1[i] * stride, a[i] * mul * w1);
+      Num<T>::store(dst + (size_t)e2[i] * stride, b[i] * mul * w2);
     }
   }
 }
@@ -207,11 +244,18 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(const T* __restrict
 JLE_API int jle_qk_prepare(const void* qkv, void* q_out, void* kv_cache, const int* positions,
                            const int* slot_mapping, const float* inv_freq, float norm_eps, float floor_scale,
                            float attn_scale, int is_bf16, int N, int Hq, int Hkv, int dh, int page_size,
-                           int write_kv, hipStream_t s) {
+                           int write_kv, int pairing, int rotary_dim, const float* norm_wq, const float* norm_wk,
+                           int norm_first, hipStream_t s) {
   if (N <= 0) return 0;
   if (dh % 2 || dh > 128 * kMaxPairsPerLane || Hq + 2 * Hkv > 65535) return JLE_BAD_ARG;
+  if (inv_freq == nullptr) rotary_dim = 0;
+  else if (rotary_dim <= 0) rotary_dim = dh;
+  if (rotary_dim % 2 || rotary_dim > dh || (pairing != 0 && pairing != 1)) return JLE_BAD_ARG;
+  // the usual case (adjacent pairs over the whole head, no weights, norm after the rotation) has a faster kernel
+  const bool usual = (inv_freq == nullptr || (pairing == 0 && rotary_dim == dh)) && norm_wq == nullptr &&
+                     norm_wk == nullptr && !norm_first;
   const bool aligned = (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)kv_cache) & 31) == 0;
-  if (aligned && dh >= 16 && dh <= 512 && (dh & (dh - 1)) == 0) {  // whatever N: a token's result is the same
+  if (usual && aligned && dh >= 16 && dh <= 512 && (dh & (dh - 1)) == 0) {  // whatever N: a token's result is the same
     const int H_here = write_kv ? Hq + 2 * Hkv : Hq;
     const int rounds = (long long)N * H_here >= 8192 ? 4 : 1;
     const int per_wave = (64 / (dh / 8)) * rounds;
@@ -234,11 +278,11 @@ JLE_API int jle_qk_prepare(const void* qkv, void* q_out, void* kv_cache, const i
   if (is_bf16)
     hipLaunchKernelGGL(qk_prepare_kernel<bf16_t>, g, b, 0, s, (const bf16_t*)qkv, (bf16_t*)q_out, (bf16_t*)kv_cache,
                        positions, slot_mapping, inv_freq, norm_eps, floor_scale, attn_scale, Hq, Hkv, dh, page_size,
-                       write_kv);
+                       write_kv, pairing, rotary_dim, norm_wq, norm_wk, norm_first);
   else
     hipLaunchKernelGGL(qk_prepare_kernel<float>, g, b, 0, s, (const float*)qkv, (float*)q_out, (float*)kv_cache,
                        positions, slot_mapping, inv_freq, norm_eps, floor_scale, attn_scale, Hq, Hkv, dh, page_size,
-                       write_kv);
+                       write_kv, pairing, rotary_dim, norm_wq, norm_wk, norm_first);
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -55,13 +55,14 @@ class StepContext:
     max_seg_len: int
     max_context_len: int
     page_size: int
-    record_routing: bool = False
-    forced_routing: Optional[dict] = None
+    # ``tap(part, name, value)``: installed by whoever wants to watch a step (tests, benchmarks).  A part may
+    # hand it named intermediate values; if the tap returns something, the part goes on with that instead.
+    tap: Optional[Any] = None
     scratch: dict = dataclasses.field(default_factory=dict)
 
 
 def build_context(ops, dtype, device, cache, entries: Sequence[StepEntry], vocab_size: int,
-                  record_routing: bool = False, forced_routing: Optional[dict] = None) -> StepContext:
+                  tap=None) -> StepContext:
     """Lays the entries end to end.  Every entry's request must hold a
     reservation for ``len(tokens)`` tokens in ``cache``."""
     ps = cache.page_size
@@ -134,5 +135,5 @@ def build_context(ops, dtype, device, cache, entries: Sequence[StepEntry], vocab
         context_lens=context_lens, state_slots=state_slots, logits_indices=logits_indices, groups=groups,
         seg_lens=seg_lens, seg_starts=seg_starts, max_seg_len=max(seg_lens),
         max_context_len=int(ctx_lens.max()), page_size=ps,
-        record_routing=record_routing, forced_routing=forced_routing,
+        tap=tap,
     )

@@ -12,7 +12,7 @@ from typing import Optional, Sequence
 
 import torch
 
-from ..cache.manager import CacheManager
+from ..cache.manager import CacheManager, pool_sizes
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .batch import StepEntry
@@ -22,19 +22,48 @@ from .scheduler import Request, Scheduler, SchedulerConfig
 
 
 class Engine:
-    def __init__(self, model, *, cache_tokens: int, page_size: int = 16, decode_batch_size: int = 64,
-                 max_num_batched_tokens: int = 2048, keep_free_pages: int = 0, reference_ops: bool = False,
-                 poison: bool = False) -> None:
-        """``cache_tokens``: tokens each layer group's page pool can hold."""
+    def __init__(self, model, *, cache_tokens: Optional[int] = None, kv_memory_fraction: Optional[float] = None,
+                 page_size: int = 16, decode_batch_size: int = 64, max_num_batched_tokens: int = 2048,
+                 max_seq_len: Optional[int] = None, keep_free_pages: int = 0, reference_ops: bool = False,
+                 poison: bool = False, decode_graphs: Optional[bool] = None) -> None:
+        """The page pools are sized either by ``cache_tokens`` (tokens that a layer group which keeps
+        every token can hold; default ``decode_batch_size * max_seq_len``) or by ``kv_memory_fraction``
+        (that part of the device memory free now, after the weights).  Groups whose retention rule
+        lets go of old tokens (chunked attention) get only what ``decode_batch_size`` requests can
+        hold of them.  ``max_seq_len``: a request ends with reason ``"length"`` when prompt and
+        output reach it; default: the configuration's ``max_position_embeddings``, if it has one.
+        ``decode_graphs``: replay steps of single tokens as recorded HIP graphs (default: on a GPU)."""
         self.model = model
         self.ops = get_ops(model.device, reference_ops=reference_ops)
-        num_pages = -(-cache_tokens // page_size)
-        self.cache = CacheManager(model.cache_needs(), page_size=page_size, num_pages=num_pages,
+        limit = getattr(getattr(model, "config", None), "max_position_embeddings", None)
+        if max_seq_len is None:
+            max_seq_len = limit
+        elif limit is not None and max_seq_len > limit:
+            raise ValueError(f"max_seq_len {max_seq_len} is beyond the model's max_position_embeddings {limit}")
+        self.max_seq_len = max_seq_len
+        needs = model.cache_needs()
+        item = torch.empty((), dtype=model.dtype).element_size()
+        memory = None
+        if kv_memory_fraction is not None:
+            if cache_tokens is not None:
+                raise ValueError("give cache_tokens or kv_memory_fraction, not both")
+            if not 0.0 < kv_memory_fraction <= 1.0 or model.device.type != "cuda":
+                raise ValueError("kv_memory_fraction must lie in (0, 1] and needs a GPU")
+            free, _ = torch.cuda.mem_get_info(model.device)
+            memory = int(free * kv_memory_fraction)
+        elif cache_tokens is None:
+            if max_seq_len is None:
+                raise ValueError("give cache_tokens, kv_memory_fraction or max_seq_len")
+            cache_tokens = decode_batch_size * max_seq_len
+        num_pages = pool_sizes(needs, page_size=page_size, itemsize=item, max_requests=decode_batch_size,
+                               max_step_tokens=max_num_batched_tokens, max_seq_len=max_seq_len,
+                               cache_tokens=cache_tokens, memory_bytes=memory)
+        self.cache = CacheManager(needs, page_size=page_size, num_pages=num_pages,
                                   max_requests=decode_batch_size, dtype=model.dtype, device=model.device,
                                   poison=poison)
-        self.runner = ModelRunner(model, self.cache, self.ops)
-        self.scheduler = Scheduler(SchedulerConfig(max_num_batched_tokens, decode_batch_size, keep_free_pages),
-                                   self.cache)
+        self.runner = ModelRunner(model, self.cache, self.ops, decode_graphs=decode_graphs)
+        self.scheduler = Scheduler(SchedulerConfig(max_num_batched_tokens, decode_batch_size, keep_free_pages,
+                                                   max_seq_len), self.cache)
         self.sampler = Sampler(self.ops, model.device)
         self._ids = itertools.count()
 
@@ -76,12 +105,17 @@ class Engine:
         the handles to pass to :meth:`decode_step` (``model.py:1243-1267``)."""
         ids = list(ids) if ids is not None else [f"req{next(self._ids)}" for _ in tokens]
         logits = self.runner.step([StepEntry(i, list(t), [len(t) - 1]) for i, t in zip(ids, tokens)])
-        return torch.argmax(logits, dim=-1).tolist(), logits, ids
+        return self._greedy(logits), logits, ids
 
     def decode_step(self, last_tokens: Sequence[int], ids: Sequence):
         """One token for each live request (``model.py:1270-1277``); returns ``(next_tokens, logits)``."""
         logits = self.runner.step([StepEntry(i, [int(t)], [0]) for i, t in zip(ids, last_tokens)])
-        return torch.argmax(logits, dim=-1).tolist(), logits
+        return self._greedy(logits), logits
+
+    def _greedy(self, logits) -> list:
+        """The largest logit of each row, lowest id among equals (the sampling kernel's greedy case)."""
+        m = logits.shape[0]
+        return self.sampler(logits, [SamplingParams()] * m, [0] * m)
 
     def release(self, ids: Sequence) -> None:
         for i in ids:

@@ -26,21 +26,21 @@ from .batch import StepEntry
 from .loading import get_ops, load_model, parse_dtype
 from .runner import ModelRunner
 
-PAGE_SIZE = 16
-MAX_LIVE_REQUESTS = 8
-
-
-def make_runner(model_dir: str, dtype, max_tokens: int, device: str = "cuda:0", page_size: int = PAGE_SIZE,
-                reference_ops: bool = False, poison: bool = False) -> ModelRunner:
+def make_runner(model_dir: str, dtype, max_tokens: int, device: str = "cuda:0", page_size: int = 16,
+                max_requests: int = 8, reference_ops: bool = False, poison: bool = False,
+                decode_graphs=None) -> ModelRunner:
+    """``max_tokens``: the most tokens live requests hold at any time, each request's count rounded
+    up to a multiple of 64; every group's pool is made for that many (plus a page per request, for
+    counts that are rounded to pages here), so pages are used again.  ``max_requests``: requests
+    that may be live at once."""
     dtype = parse_dtype(dtype)
     ops = get_ops(device, reference_ops=reference_ops)
     model = load_model(model_dir, dtype, device)
-    # every group gets pages for max_tokens tokens, each request's count rounded up to whole pages
     rounded = -(-max_tokens // 64) * 64
-    num_pages = rounded // page_size + MAX_LIVE_REQUESTS
+    num_pages = -(-rounded // page_size) + max_requests
     cache = CacheManager(model.cache_needs(), page_size=page_size, num_pages=num_pages,
-                         max_requests=MAX_LIVE_REQUESTS, dtype=dtype, device=device, poison=poison)
-    return ModelRunner(model, cache, ops)
+                         max_requests=max_requests, dtype=dtype, device=device, poison=poison)
+    return ModelRunner(model, cache, ops, decode_graphs=decode_graphs)
 
 
 def replay(runner: ModelRunner, lines, out_dir: str, out=sys.stdout) -> None:
@@ -72,9 +72,13 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--device", default="cuda:0")
-    ap.add_argument("--page-size", type=int, default=PAGE_SIZE)
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--max-requests", type=int, default=8, help="requests that may be live at once")
+    ap.add_argument("--no-decode-graphs", action="store_true",
+                    help="run steps of single tokens launch by launch instead of replaying recorded HIP graphs")
     args = ap.parse_args(argv)
-    runner = make_runner(args.model, args.dtype, args.max_tokens, args.device, args.page_size)
+    runner = make_runner(args.model, args.dtype, args.max_tokens, args.device, args.page_size, args.max_requests,
+                         decode_graphs=False if args.no_decode_graphs else None)
     replay(runner, sys.stdin, args.out)
     return 0
 

@@ -18,22 +18,23 @@ from .batch import StepEntry, build_context
 
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager, ops) -> None:
+    def __init__(self, model, cache: CacheManager, ops, decode_graphs: Optional[bool] = None) -> None:
         self.model = model
         self.cache = cache
         self.ops = ops
+        self.decode_graphs = decode_graphs
         self.steps_run = 0
         self.tokens_run = 0
 
     @torch.no_grad()
-    def step(self, entries: Sequence[StepEntry], *, record_routing: bool = False,
-             forced_routing: Optional[dict] = None) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], *, tap=None) -> torch.Tensor:
         """Runs only the tokens it is given.  A request not yet known to the
         cache is added.  Pages for the new tokens are taken first (for all
         entries or for none: :class:`OutOfPages` leaves the cache unchanged);
         after the model has run, the tokens are counted and pages that a
         retention rule has passed are given back.  Returns ``[wanted, vocab]``
-        float32, in the order of the entries and of each entry's ``want``."""
+        float32, in the order of the entries and of each entry's ``want``.  ``tap``: see
+        :class:`~.batch.StepContext`."""
         cache = self.cache
         seen = set()
         for e in entries:
@@ -56,7 +57,7 @@ class ModelRunner:
             raise
         try:
             ctx = build_context(self.ops, self.model.dtype, self.model.device, cache, entries,
-                                self.model.plan.vocab_size, record_routing, forced_routing)
+                                self.model.plan.vocab_size, tap)
             logits = self.model.forward(ctx, cache)
         except Exception:
             for rid in reserved:

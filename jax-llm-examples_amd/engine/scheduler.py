@@ -4,7 +4,8 @@ under a token budget, decodes, finishes and frees.
 The reference's serving loop (``serving/serving_jax/serving_loop.py``) keeps a fixed
 number of decode slots (``decode_batch_size``, ``:422-434``), prefills whole prompts
 in their own batches (``:697-758``), lets decode go first (``:794-795``), finishes a
-request on an EOS token or after ``max_decode_length`` tokens (``:656-660``), and has
+request on an EOS token or after ``max_decode_length`` tokens (``:656-660``; here also when
+prompt and output reach ``max_seq_len``, the configuration's context limit), and has
 no answer to a full cache.  Here one step holds decode tokens of running
 requests beside portions of prompts; the option names ``decode_batch_size``,
 ``max_decode_length`` and ``eos_tokens`` keep the reference's meaning.
@@ -35,6 +36,7 @@ class SchedulerConfig:
     max_num_batched_tokens: int = 2048  # tokens one step may hold
     decode_batch_size: int = 64  # requests that may be running at once
     keep_free_pages: int = 0  # pages per group that admitting a new request must leave free
+    max_seq_len: Optional[int] = None  # a request ends when its prompt and output together reach this many tokens
 
 
 @dataclasses.dataclass
@@ -97,6 +99,11 @@ class Scheduler:
     def add(self, request: Request) -> None:
         if not request.prompt:
             raise ValueError(f"request {request.id!r} has an empty prompt")
+        limit = self.cfg.max_seq_len
+        if limit is not None and len(request.prompt) > limit:
+            # the reference asserts the same of a prompt (llama4/llama4_jax/model.py:1248)
+            raise ValueError(f"request {request.id!r}: a prompt of {len(request.prompt)} tokens is longer than "
+                             f"max_seq_len {limit}")
         request.state = WAITING
         self.waiting.append(request)
 
@@ -215,6 +222,8 @@ class Scheduler:
                 self._finish(r, "eos")
             elif len(r.output) >= p.max_decode_length:
                 self._finish(r, "length")
+            elif self.cfg.max_seq_len is not None and len(r.prompt) + len(r.output) >= self.cfg.max_seq_len:
+                self._finish(r, "length")  # the context limit: there is no position for a further token
             if r.state == FINISHED:
                 finished.append(r)
         return finished

@@ -58,6 +58,13 @@ def main(argv=None) -> int:
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048, help="token budget of one step")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--cache-tokens", type=int, help="tokens the page pools hold (default: batch size x max-seq-len)")
+    ap.add_argument("--num-pages", type=int, help="the same in pages of --page-size tokens")
+    ap.add_argument("--kv-memory-fraction", type=float,
+                    help="size the page pools to this part of the device memory that is free after the weights")
+    ap.add_argument("--no-decode-graphs", action="store_true",
+                    help="run steps of single tokens launch by launch instead of replaying recorded HIP graphs")
+    ap.add_argument("--profile", metavar="DIR",
+                    help="trace the generation with the PyTorch profiler: a kernel table on stderr, a trace file in DIR")
     ap.add_argument("--sample-temp", type=float, default=0.0, help="0 = greedy")
     ap.add_argument("--sample-topk", type=int, default=0, help="sample among the k most likely tokens (0 = all)")
     ap.add_argument("--sample-seed", type=int, default=0)
@@ -90,17 +97,38 @@ def main(argv=None) -> int:
         raise SystemExit("give --ckpt-path or --random-weights")
 
     prompts = _parse_prompts(args, model.plan.vocab_size)
-    cache_tokens = args.cache_tokens or args.decode_batch_size * args.max_seq_len
-    engine = Engine(model, cache_tokens=cache_tokens, page_size=args.page_size,
-                    decode_batch_size=args.decode_batch_size, max_num_batched_tokens=args.max_num_batched_tokens)
+    limit = getattr(getattr(model, "config", None), "max_position_embeddings", None)
+    max_seq_len = args.max_seq_len if limit is None else min(args.max_seq_len, limit)
+    sizing = {}
+    if args.kv_memory_fraction is not None:
+        sizing["kv_memory_fraction"] = args.kv_memory_fraction
+    else:
+        sizing["cache_tokens"] = (args.cache_tokens or (args.num_pages or 0) * args.page_size
+                                  or args.decode_batch_size * max_seq_len)
+    engine = Engine(model, page_size=args.page_size, decode_batch_size=args.decode_batch_size,
+                    max_num_batched_tokens=args.max_num_batched_tokens, max_seq_len=max_seq_len,
+                    decode_graphs=False if args.no_decode_graphs else None, **sizing)
     eos = tuple(int(t) for t in args.eos_tokens.split(",") if t)
     params = [SamplingParams(sample_temp=args.sample_temp, sample_topk=args.sample_topk,
                              seed=args.sample_seed + i, max_decode_length=args.max_decode_length, eos_tokens=eos)
               for i in range(len(prompts))]
     t0 = time.time()
-    outs = engine.generate(prompts, params)
-    if model.device.type == "cuda":
-        torch.cuda.synchronize()
+    if args.profile:
+        import os
+
+        from torch.profiler import ProfilerActivity, profile
+
+        os.makedirs(args.profile, exist_ok=True)
+        with profile(activities=[ProfilerActivity.CPU, ProfilerActivity.CUDA]) as prof:
+            outs = engine.generate(prompts, params)
+            if model.device.type == "cuda":
+                torch.cuda.synchronize()
+        prof.export_chrome_trace(os.path.join(args.profile, "generate_trace.json"))
+        print(prof.key_averages().table(sort_by="cuda_time_total", row_limit=25), file=sys.stderr)
+    else:
+        outs = engine.generate(prompts, params)
+        if model.device.type == "cuda":
+            torch.cuda.synchronize()
     dt = time.time() - t0
     for i, o in enumerate(outs):
         print(json.dumps({"prompt": i, "tokens": o}))

@@ -24,7 +24,8 @@ _SIGNATURES = {
     "jle_gather_rows": [_vp, _vp, _vp, _i, _i, _vp],
     "jle_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
     "jle_moe_combine": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
-    "jle_qk_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_qk_prepare": [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _f, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i,
+                       _vp],
     "jle_paged_attention_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
                                     _vp, _vp],
     "jle_moe_route": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
@@ -315,14 +316,27 @@ class HipOps:
         return out
 
     # ------------------------------------------------------------------ attention
-    def qk_prepare_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, positions, inv_freq, qk_norm_eps,
-                            query_scale, kv_cache, slot_mapping):
+    def qk_prepare_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, positions, prep, kv_cache, slot_mapping):
+        """``prep``: a :class:`~..parts.base.QKPreparation`."""
         n = qkv.shape[0]
         hq, hk, dh = num_heads, num_kv_heads, head_dim
         self._chk(qkv, None, (n, (hq + 2 * hk) * dh), "q|k|v")
         self._chk(positions, torch.int32, (n,), "positions")
-        if inv_freq is not None:
-            self._chk(inv_freq, torch.float32, (dh // 2,), "inv_freq")
+        rot = prep.rotation
+        inv_freq, pairing, rd = None, 0, 0
+        if rot is not None:
+            inv_freq, rd = rot.inv_freq, int(rot.rotary_dim) or dh
+            if rot.pairing not in ("adjacent", "half"):
+                raise KernelError(f"rotary/norm kernel: unknown pairing {rot.pairing!r}")
+            pairing = 0 if rot.pairing == "adjacent" else 1
+            if rd % 2 or not 0 < rd <= dh:
+                raise KernelError(f"rotary/norm kernel: {rd} rotated elements of a head of {dh}")
+            self._chk(inv_freq, torch.float32, (rd // 2,), "inv_freq")
+        for w, what in ((prep.norm_weight_q, "q norm weight"), (prep.norm_weight_k, "k norm weight")):
+            if w is not None:
+                if prep.norm_eps is None:
+                    raise KernelError("rotary/norm kernel: norm weights without a norm")
+                self._chk(w, torch.float32, (dh,), what)
         ps = 0
         if kv_cache is not None:
             ps = kv_cache.shape[3]
@@ -331,11 +345,12 @@ class HipOps:
         if dh % 2 or dh > 512:
             raise KernelError(f"rotary/norm kernel: head size {dh} must be even and at most 512")
         q = torch.empty(n, hq, dh, dtype=qkv.dtype, device=qkv.device)
-        fs, sc = (query_scale if query_scale is not None else (0.0, 0.0))
+        fs, sc = (prep.query_scale if prep.query_scale is not None else (0.0, 0.0))
         self._call("jle_qk_prepare", _p(qkv), _p(q), _p(kv_cache), _p(positions),
                    _p(slot_mapping) if kv_cache is not None else None, _p(inv_freq),
-                   -1.0 if qk_norm_eps is None else float(qk_norm_eps), float(fs), float(sc), self._is_bf16(qkv),
-                   n, hq, hk, dh, max(ps, 1), 0 if kv_cache is None else 1)
+                   -1.0 if prep.norm_eps is None else float(prep.norm_eps), float(fs), float(sc), self._is_bf16(qkv),
+                   n, hq, hk, dh, max(ps, 1), 0 if kv_cache is None else 1, pairing, rd, _p(prep.norm_weight_q),
+                   _p(prep.norm_weight_k), int(bool(prep.norm_first)))
         return q
 
     PREFILL_TILE = 32  # tokens per prefill work item (the kernels take 16 or 32)

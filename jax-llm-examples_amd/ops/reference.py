@@ -79,48 +79,53 @@ class ReferenceOps:
         return (torch.nn.functional.silu(g) * u).to(gate_up.dtype)
 
     # ------------------------------------------------------------------ attention
-    def qk_prepare_kv_write(
-        self,
-        qkv,
-        num_heads: int,
-        num_kv_heads: int,
-        head_dim: int,
-        positions,
-        inv_freq: Optional[torch.Tensor],
-        qk_norm_eps: Optional[float],
-        query_scale: Optional[tuple],
-        kv_cache: Optional[torch.Tensor],
-        slot_mapping: Optional[torch.Tensor],
-    ):
-        """Splits fused q|k|v rows, rotates q and k by interleaved pairs
-        (angle ``pos * inv_freq[j]`` in float32), L2-normalises q and k over the
-        head (no weight) if ``qk_norm_eps`` is given, multiplies q by
-        ``1 + attn_scale * ln(1 + floor((pos + 1) / floor_scale))`` if
-        ``query_scale = (floor_scale, attn_scale)``, and writes k and v into their page at
-        ``slot = page * page_size + offset``.  ``kv_cache`` is ``[pages, 2, kv_heads, page_size *
-        head_dim]`` in memory: plane 0 holds keys as ``[page_size, head_dim]``, plane 1 holds values
-        transposed, ``[head_dim, page_size]``.  Returns q ``[N, num_heads, head_dim]``."""
+    def qk_prepare_kv_write(self, qkv, num_heads: int, num_kv_heads: int, head_dim: int, positions, prep,
+                            kv_cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]):
+        """Splits fused q|k|v rows and prepares q and k as ``prep`` (a
+        :class:`~..parts.base.QKPreparation`) says: the rotation turns element pairs by the angle
+        ``pos * inv_freq[j]`` (float32) - adjacent pairs ``(x[2j], x[2j+1])`` or half-split pairs
+        ``(x[j], x[j + rotary_dim/2])`` of the leading ``rotary_dim`` elements; the RMS norm over the
+        head (``x / sqrt(mean(x^2) + eps)``, times a weight if there is one) comes after the rotation,
+        or before it with ``norm_first``; ``query_scale = (floor_scale, attn_scale)`` multiplies q by
+        ``1 + attn_scale * ln(1 + floor((pos + 1) / floor_scale))``.  Then k and v are written into
+        their page at ``slot = page * page_size + offset``.  ``kv_cache`` is ``[pages, 2, kv_heads,
+        page_size * head_dim]`` in memory: plane 0 holds keys as ``[page_size, head_dim]``, plane 1
+        holds values transposed, ``[head_dim, page_size]``.  Returns q ``[N, num_heads, head_dim]``."""
         n = qkv.shape[0]
         dt = qkv.dtype
         hq, hk, dh = num_heads, num_kv_heads, head_dim
         q = qkv[:, : hq * dh].float().reshape(n, hq, dh)
         k = qkv[:, hq * dh : (hq + hk) * dh].float().reshape(n, hk, dh)
         v = qkv[:, (hq + hk) * dh :].float().reshape(n, hk, dh)
-        if inv_freq is not None:
-            ang = positions.float()[:, None] * inv_freq.float()[None, :]
+
+        def norm(x, w):
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + prep.norm_eps)
+            return x if w is None else x * w.float()
+
+        if prep.norm_eps is not None and prep.norm_first:
+            q, k = norm(q, prep.norm_weight_q), norm(k, prep.norm_weight_k)
+        rot = prep.rotation
+        if rot is not None:
+            rd = int(rot.rotary_dim) or dh
+            ang = positions.float()[:, None] * rot.inv_freq.float()[None, :]
             sin, cos = torch.sin(ang)[:, None, :], torch.cos(ang)[:, None, :]
 
-            def rot(x):
-                x = x.reshape(n, -1, dh // 2, 2)
-                a, b = x[..., 0], x[..., 1]
-                return torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1).reshape(n, -1, dh)
+            def turn(x):
+                head, rest = x[..., :rd], x[..., rd:]
+                if rot.pairing == "adjacent":
+                    pairs = head.reshape(n, -1, rd // 2, 2)
+                    a, b = pairs[..., 0], pairs[..., 1]
+                    head = torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1).reshape(n, -1, rd)
+                else:
+                    a, b = head[..., : rd // 2], head[..., rd // 2:]
+                    head = torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1)
+                return torch.cat([head, rest], dim=-1)
 
-            q, k = rot(q), rot(k)
-        if qk_norm_eps is not None:
-            q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + qk_norm_eps)
-            k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + qk_norm_eps)
-        if query_scale is not None:
-            floor_scale, attn_scale = query_scale
+            q, k = turn(q), turn(k)
+        if prep.norm_eps is not None and not prep.norm_first:
+            q, k = norm(q, prep.norm_weight_q), norm(k, prep.norm_weight_k)
+        if prep.query_scale is not None:
+            floor_scale, attn_scale = prep.query_scale
             s = 1.0 + attn_scale * torch.log1p(torch.floor((positions.float() + 1.0) / floor_scale))
             q = q * s[:, None, None]
         if kv_cache is not None:

@@ -55,6 +55,23 @@ class Part:
     def finalize(self) -> None:
         """Called once after all parameters are filled."""
 
+    # A part whose ``forward`` only launches work on the current stream (no copy to the host, no size that
+    # depends on values on the device) may be recorded into a HIP graph of the decode step.  Parts that do not
+    # say so are always run step by step.
+    graph_safe = False
+
+    # ------------------------------------------------------------------ what a step costs (for rooflines)
+    def step_weight_bytes(self, observed=None) -> int:
+        """Bytes of parameters that one step has to read, each once.  ``observed``: what this part
+        handed to the step's tap (see :class:`~..engine.batch.StepContext`), if a tap was installed
+        and the part offers something; a part that reads only some of its parameters (routed
+        experts) counts from it."""
+        return sum(t.numel() * t.element_size() for t in self.params.values())
+
+    def flops_per_token(self) -> float:
+        """Floating-point operations of the part's matrix products for one token."""
+        return 2.0 * sum(t.numel() for t in self.params.values() if t.dim() >= 2)
+
 
 # --------------------------------------------------------------------------- cache needs
 @dataclasses.dataclass(frozen=True)
@@ -62,6 +79,7 @@ class CacheNeed:
     """What one run of a mixer needs from the cache manager.
 
     ``kv``: ``None`` or ``(num_kv_heads, head_dim)``, keys and values per token.
+    ``paged``: further per-token tensors in pages (see below).
     ``retention``: which earlier tokens a query at position ``p`` may still read:
     ``("all",)``; ``("chunk", C)``: those with ``pos >= (p // C) * C``;
     ``("window", W)``: those with ``pos > p - W``.  Pages that hold only
@@ -73,6 +91,13 @@ class CacheNeed:
     retention: tuple = ("all",)
     state_shape: Optional[tuple[int, ...]] = None
     state_dtype: Optional[torch.dtype] = None
+    # Other things kept per token, in pages of their own under the same retention rule: a tuple of
+    # ``(name, per-token shape)`` pairs, e.g. ``(("latent", (96,)),)`` or keys and values of different
+    # sizes ``(("k", (2, 24)), ("v", (2, 8)))``.  Each becomes a tensor ``[pages, page_size, *shape]`` in the
+    # run dtype that the mixer reads and writes through its block table and slot mapping
+    # (``CacheView.pages[name]``).  ``kv`` is the layout the attention kernels read (keys ``[page_size,
+    # head_dim]`` and values transposed in one tensor).
+    paged: tuple = ()
 
 
 def first_needed_position(retention: tuple, next_pos: int) -> int:
@@ -102,6 +127,11 @@ class Mixer(Part):
     def cache_need(self) -> CacheNeed:
         return CacheNeed()
 
+    def mixing_flops(self, start: int, count: int) -> float:
+        """Floating-point operations of moving information between positions (beyond the matrix
+        products of :meth:`flops_per_token`) for ``count`` tokens of one request from position ``start``."""
+        return 0.0
+
     def forward(self, h: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:  # pragma: no cover
         raise NotImplementedError
 
@@ -126,16 +156,52 @@ class Norm(Part):
         raise NotImplementedError
 
 
+@dataclasses.dataclass
+class Rotation:
+    """A rotary encoding as data: element pairs of a head are turned by ``pos * inv_freq[j]``.
+
+    ``inv_freq``: float32 ``[rotary_dim / 2]``; the angles are formed in float32 inside the kernel.
+    ``pairing``: ``"adjacent"`` pairs ``(x[2j], x[2j+1])``; ``"half"`` pairs ``(x[j], x[j + rotary_dim/2])``.
+    ``rotary_dim``: the leading elements of a head that are rotated (the rest pass unchanged)."""
+
+    inv_freq: torch.Tensor
+    pairing: str = "adjacent"
+    rotary_dim: int = 0
+
+
+@dataclasses.dataclass
+class QKPreparation:
+    """What happens to the q and k rows of an attention mixer between the projection and the
+    scores, as data the preparation kernel takes: the rotation (from the position encoding), an
+    RMS norm over the head with or without weights, before or after the rotation, and a
+    position-dependent scale of the queries."""
+
+    rotation: Optional[Rotation] = None
+    norm_eps: Optional[float] = None  # None: no norm
+    norm_weight_q: Optional[torch.Tensor] = None  # float32 [head_dim]; None: weightless
+    norm_weight_k: Optional[torch.Tensor] = None
+    norm_first: bool = False  # the norm comes before the rotation
+    query_scale: Optional[tuple] = None  # (floor_scale, attn_scale): q *= 1 + attn_scale * ln(1 + floor((pos + 1) / floor_scale))
+
+    @property
+    def plain(self) -> bool:
+        """The case every kernel takes: adjacent pairs over the whole head, weightless norm after the rotation."""
+        r = self.rotation
+        return ((r is None or (r.pairing == "adjacent" and r.rotary_dim in (0, 2 * r.inv_freq.numel())))
+                and self.norm_weight_q is None and self.norm_weight_k is None and not self.norm_first)
+
+
 class PositionEncoding:
-    """Turns integer positions into what the mixer's kernels take.  For rotary
-    kinds that is ``inv_freq`` (float32 ``[head_dim/2]``), from which angles
-    ``pos * inv_freq`` are formed in float32 inside the kernel."""
+    """Turns integer positions into what the mixer's kernels take.  Rotary kinds return a
+    :class:`Rotation` from :meth:`rotation` (frequencies, which elements pair up, how many are
+    rotated); the attention mixer hands it to the kernel that prepares q and k.  Another family
+    (additive, learned) is applied by the mixer that names it."""
 
     def __init__(self, spec: PartSpec, head_dim: int) -> None:
         self.spec = spec
         self.head_dim = head_dim
 
-    def inv_freq(self) -> Optional[torch.Tensor]:
+    def rotation(self) -> Optional[Rotation]:
         return None
 
 

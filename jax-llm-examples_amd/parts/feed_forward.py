@@ -29,6 +29,8 @@ class DenseSwiGLU(FeedForward):
             "w_down": ParamSpec((self.hidden, self.inter)),
         }
 
+    graph_safe = True
+
     def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
         ops = ctx.ops
         return ops.linear(ops.swiglu_linear(h, self.params["w_gate_up"]), self.params["w_down"])
@@ -45,7 +47,6 @@ class MoESigmoidShared(FeedForward):
         self.top_k = int(spec.top_k)
         self.inter = int(spec.intermediate_size)
         self.shared_inter = int(spec.get("shared_intermediate_size") or 0)
-        self.last_routing = None  # (expert ids, gates) of the latest call, for tests
         self.tiled = False  # expert matrices are in the kernels' streaming layout (ops/layout.py)
 
     def param_specs(self):
@@ -60,6 +61,24 @@ class MoESigmoidShared(FeedForward):
             specs["shared_down"] = ParamSpec((d, self.shared_inter))
         return specs
 
+    graph_safe = True
+
+    def step_weight_bytes(self, observed=None) -> int:
+        """Of the routed experts only those that some token of the step chose (``observed``: the
+        ``(expert ids, gates)`` this part handed to the step's tap; without it, all)."""
+        n = self.num_experts if observed is None else int(torch.unique(observed[0]).numel())
+        total = 0
+        for name, t in self.params.items():
+            b = t.numel() * t.element_size()
+            total += b // self.num_experts * n if name in ("w_gate_up", "w_down") else b
+        return total
+
+    def flops_per_token(self) -> float:
+        per = 0
+        for name, t in self.params.items():
+            per += t.numel() // self.num_experts * self.top_k if name in ("w_gate_up", "w_down") else t.numel()
+        return 2.0 * per
+
     def finalize(self) -> None:
         from ..ops.layout import can_tile, tile_
 
@@ -72,12 +91,12 @@ class MoESigmoidShared(FeedForward):
     def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
         ops = ctx.ops
         expert_ids, gates, grouping = ops.moe_route(h32, self.params["router"], self.top_k, group=True)
-        if ctx.record_routing:
-            self.last_routing = (expert_ids.clone(), gates.clone())
-        forced = ctx.forced_routing.get(id(self)) if ctx.forced_routing else None
-        if forced is not None:
-            expert_ids, gates = forced
-            grouping = None
+        tap = getattr(ctx, "tap", None)
+        if tap is not None:  # whoever watches the step sees the choice and may replace it
+            replaced = tap(self, "routing", (expert_ids, gates))
+            if replaced is not None:
+                expert_ids, gates = replaced
+                grouping = None
         shared = (self.params["shared_gate_up"], self.params["shared_down"]) if self.shared_inter else None
         return ops.moe_experts(h, expert_ids, gates, self.params["w_gate_up"], self.params["w_down"],
                                shared_weights=shared, tiled=self.tiled, grouping=grouping)

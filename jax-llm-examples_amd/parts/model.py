@@ -103,7 +103,8 @@ class DecoderModel:
             view = CacheView(cache_id=e.cache, writes=e.writes_cache, group=gi, state=cache.state.get(e.cache))
             if gi is not None:
                 g = ctx.groups[gi]
-                view.kv = cache.groups[gi].tensors[e.cache]
+                view.kv = cache.groups[gi].tensors.get(e.cache)
+                view.pages = cache.groups[gi].pages.get(e.cache)
                 view.block_table = g.block_table
                 view.slot_mapping = g.slot_mapping
                 view.attn_meta = g

@@ -13,6 +13,8 @@ class RMSNorm(Norm):
         self.weighted = bool(spec.get("weighted", True))
         self.size = spec.get("size")
 
+    graph_safe = True
+
     def param_specs(self):
         if not self.weighted:
             return {}

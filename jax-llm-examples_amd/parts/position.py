@@ -5,8 +5,8 @@
 ``theta ** -(2j / head_dim)`` (``model.py:706-708``) and, if the configuration has
 ``rope_scaling``, the llama3 correction (``model.py:654-672``).  Angles are formed
 in float32 from integer positions inside the kernel (``model.py:710-718``: a
-reduced-precision product here is catastrophic); this part only provides
-``inv_freq``.
+reduced-precision product here is catastrophic); this part says, as data, which
+frequencies there are, which elements pair up and how many of a head are rotated.
 """
 from __future__ import annotations
 
@@ -15,7 +15,7 @@ from typing import Optional
 
 import torch
 
-from .base import PositionEncoding, register_position
+from .base import PositionEncoding, Rotation, register_position
 
 
 @register_position("none")
@@ -57,3 +57,6 @@ class RopeInterleaved(PositionEncoding):
                 int(scaling["original_max_position_embeddings"]),
             )
         return inv.to(torch.float32)
+
+    def rotation(self) -> Rotation:
+        return Rotation(self.inv_freq(), pairing="adjacent", rotary_dim=self.head_dim)

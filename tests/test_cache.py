@@ -154,3 +154,65 @@ def test_pages_needed_matches_what_reserve_takes():
         assert [b - a for a, b in zip(m.num_free_pages(), before)] == need
         m.commit("a")
     assert m.pages_needed_new(17) == [3, 3, 3]
+
+
+def test_each_group_is_sized_by_what_its_retention_rule_can_hold():
+    """A group that lets go of old tokens needs a chunk plus a step's portion per request, whatever the
+    context length; sized for the whole context it would take most of the memory for nothing."""
+    from jax_llm_examples_amd.cache import pool_sizes, tokens_held_at_most
+
+    # three chunked runs per run that keeps everything, as in the large configuration
+    needs = {i: CacheNeed(kv=(8, 128), retention=("all",) if i % 4 == 3 else ("chunk", 8192)) for i in range(8)}
+    kw = dict(page_size=16, itemsize=2, max_requests=4, max_step_tokens=2048)
+    assert tokens_held_at_most(("chunk", 8192), 2048, None) == 10240
+    assert tokens_held_at_most(("window", 100), 7, 60) == 60 and tokens_held_at_most(("all",), 7, None) is None
+    sizes = pool_sizes(needs, cache_tokens=4 * 32768, **kw)
+    chunked, full = sizes[0], sizes[1]  # groups in order of their first run
+    assert full == 4 * 32768 // 16
+    assert chunked == 4 * (10240 // 16 + 1) and chunked < full // 3
+    # the same memory holds many more tokens of context than with equal pools
+    page = 2 * 8 * 128 * 16 * 2
+    equal_pools_bytes = 8 * page * full
+    budget = equal_pools_bytes // 2
+    by_memory = pool_sizes(needs, memory_bytes=budget, **kw)
+    assert by_memory[0] == chunked and by_memory[1] * 16 > 32768 * 4
+    used = 6 * page * by_memory[0] + 2 * page * by_memory[1]
+    assert used <= budget < used + 2 * page  # the largest that fits
+    with pytest.raises(ValueError, match="one page"):
+        pool_sizes(needs, memory_bytes=100, **kw)
+    # a manager built with these sizes: a request of 32,768 tokens fits, fed in portions
+    small = {0: CacheNeed(kv=(1, 8), retention=("chunk", 64)), 1: CacheNeed(kv=(1, 8), retention=("all",))}
+    sz = pool_sizes(small, page_size=8, itemsize=4, max_requests=2, max_step_tokens=24, cache_tokens=2 * 1000)
+    assert sz == {0: 2 * (88 // 8 + 1), 1: 250}
+    m = CacheManager(small, page_size=8, num_pages=sz, max_requests=2, dtype=torch.float32, device="cpu")
+    for rid in ("a", "b"):
+        m.add_request(rid)
+    for step in range(41):
+        for rid in ("a", "b"):
+            m.reserve(rid, 24)  # never out of pages in the small pool
+        for rid in ("a", "b"):
+            m.commit(rid)
+        m.check()
+    assert m.num_tokens("a") == 984 and m.groups[0].pool.handed_out > m.groups[0].pool.num_pages
+
+
+def test_further_per_token_tensors_get_pages_of_their_own_shapes():
+    needs = {0: CacheNeed(kv=(2, 8), retention=("all",)),
+             1: CacheNeed(paged=(("k", (2, 24)), ("v", (2, 8))), retention=("all",)),
+             2: CacheNeed(paged=(("latent", (10,)),), retention=("window", 5)),
+             3: CacheNeed(paged=(("k", (2, 24)), ("v", (2, 8))), retention=("all",))}
+    m = CacheManager(needs, page_size=4, num_pages={0: 6, 1: 5, 2: 3}, max_requests=2, dtype=torch.bfloat16,
+                     device="cpu", poison=True)
+    assert [g.cache_ids for g in m.groups] == [[0], [1, 3], [2]]
+    assert m.groups[1].pages[3]["k"].shape == (5, 4, 2, 24) and m.groups[1].pages[1]["v"].shape == (5, 4, 2, 8)
+    assert m.groups[2].pages[2]["latent"].shape == (3, 4, 10) and not m.groups[2].tensors
+    assert m.groups[1].bytes_per_token() == 2 * (48 + 16) * 2 and m.groups[2].bytes_per_token() == 20
+    assert m.bytes_per_token() == 2 * 2 * 8 * 2 + 256 + 20
+    m.add_request("a")
+    m.reserve("a", 9)
+    page = m.table("a", 2)[0]
+    m.groups[2].pages[2]["latent"][page] = 1.0
+    m.commit("a")  # the window has passed the first page: given back and poisoned
+    assert m.table("a", 2)[0] == -1 and bool(m.groups[2].pages[2]["latent"][page].isnan().all())
+    m.free("a")
+    m.check()

@@ -102,3 +102,13 @@ def test_scout_preset_matches_the_benchmark_configuration():
         (16, 8192, 16384, 202048)
     assert cfg.rope_scaling.factor == 16 and sum(cfg.no_rope_layers) == 36 and len(cfg.moe_layers) == 48
     assert len(Llama4TextConfig.from_dict(preset("llama4-maverick", 8)).moe_layers) == 4
+
+
+def test_floor_scale_is_written_as_the_integer_it_is():
+    """Checkpoints store a whole number there, and strict readers of config.json refuse ``8192.0``."""
+    top = tiny_config_json("A")
+    cfg = Llama4TextConfig.from_dict(top)
+    out = cfg.to_dict()
+    assert isinstance(out["floor_scale"], int) and out["floor_scale"] == 16
+    top["floor_scale"] = 2.5
+    assert Llama4TextConfig.from_dict(top).to_dict()["floor_scale"] == 2.5

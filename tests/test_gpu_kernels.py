@@ -92,15 +92,22 @@ def test_qk_prepare_of_a_token_does_not_depend_on_the_batch(ops, ref, dt):
     qkv, pos, pages, slots, inv_freq = _prep_case(hq, hk, dh, n, ps, dt)
     c1 = torch.zeros(pages, 2, hk, ps, dh, dtype=dt, device=DEV)
     c2, c3 = c1.clone(), c1.clone()
-    q1 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq, 1e-5, (16.0, 0.1), c1, slots)
-    q2 = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq, 1e-5, (16.0, 0.1), c2, slots)
+    q1 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv_freq, 1e-5, (16.0, 0.1)), c1, slots)
+    q2 = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv_freq, 1e-5, (16.0, 0.1)), c2, slots)
     assert torch.allclose(q1.float(), q2.float(), **_tol(dt)) and torch.allclose(c1.float(), c2.float(), **_tol(dt))
     few = slice(100, 107)
-    q3 = ops.qk_prepare_kv_write(qkv[few].contiguous(), hq, hk, dh, pos[few].contiguous(), inv_freq, 1e-5,
-                                 (16.0, 0.1), c3, slots[few].contiguous())
+    q3 = ops.qk_prepare_kv_write(qkv[few].contiguous(), hq, hk, dh, pos[few].contiguous(),
+                                 _prep(inv_freq, 1e-5, (16.0, 0.1)), c3, slots[few].contiguous())
     assert torch.equal(q3, q1[few])
     written = c3 != 0
     assert written.any() and torch.equal(c3[written], c1[written])
+
+
+def _prep(inv_freq=None, eps=None, qs=None, **kw):
+    from jax_llm_examples_amd.parts.base import QKPreparation, Rotation
+
+    rot = None if inv_freq is None else Rotation(inv_freq, kw.pop("pairing", "adjacent"), kw.pop("rotary_dim", 0))
+    return QKPreparation(rotation=rot, norm_eps=eps, query_scale=qs, **kw)
 
 
 def _prep_case(hq, hk, dh, n, ps, dt, seed=0):
@@ -121,14 +128,40 @@ def test_qk_prepare_kv_write(ops, ref, dt, hq, hk, dh):
                           (True, 1e-3, (4.0, 0.3))]:
         c1 = torch.zeros(pages, 2, hk, ps, dh, dtype=dt, device=DEV)
         c2 = c1.clone()
-        q1 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq if rope else None, eps, qs, c1, slots)
-        q2 = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq if rope else None, eps, qs, c2, slots)
+        q1 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv_freq if rope else None, eps, qs), c1, slots)
+        q2 = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv_freq if rope else None, eps, qs), c2, slots)
         assert torch.allclose(q1.float(), q2.float(), **_tol(dt))
         assert torch.allclose(c1.float(), c2.float(), **_tol(dt))
         assert (c1[:, 1] != 0).any() and torch.equal(c1 == 0, c2 == 0)  # wrote exactly the same places
-    q3 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq, None, None, None, None)  # a run that only reads
-    assert torch.allclose(q3.float(), ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, inv_freq, None, None, None,
+    q3 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv_freq), None, None)  # a run that only reads
+    assert torch.allclose(q3.float(), ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv_freq), None,
                                                                None).float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("hq,hk,dh,rd", [(4, 2, 32, 32), (5, 1, 48, 16), (40, 8, 128, 64), (6, 2, 80, 80)])
+def test_qk_prepare_other_rotations_and_norms(ops, ref, dt, hq, hk, dh, rd):
+    """What Llama 4 does not use but the preparation takes as data: half-split pairs, a rotation of the
+    head's leading part only, norm weights, the norm before the rotation."""
+    n, ps = 11, 8
+    qkv, pos, pages, slots, _ = _prep_case(hq, hk, dh, n, ps, dt, seed=3)
+    inv = (1.0 / (10000.0 ** (torch.arange(0, rd, 2).float() / rd))).to(DEV)
+    wq, wk = _rand(dh, seed=7) + 1.5, _rand(dh, seed=8) - 1.5
+    cases = [dict(pairing="half", rotary_dim=rd), dict(pairing="adjacent", rotary_dim=rd),
+             dict(pairing="half", rotary_dim=rd, eps=1e-4, norm_weight_q=wq, norm_weight_k=wk),
+             dict(pairing="adjacent", rotary_dim=rd, eps=1e-4, norm_weight_q=wq, norm_weight_k=wk, norm_first=True),
+             dict(pairing="half", rotary_dim=rd, eps=1e-2, norm_first=True, qs=(4.0, 0.3))]
+    for kw in cases:
+        c1 = torch.zeros(pages, 2, hk, ps, dh, dtype=dt, device=DEV)
+        c2 = c1.clone()
+        q1 = ops.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv, **dict(kw)), c1, slots)
+        q2 = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv, **dict(kw)), c2, slots)
+        assert torch.allclose(q1.float(), q2.float(), **_tol(dt)), kw
+        assert torch.allclose(c1.float(), c2.float(), **_tol(dt)), kw
+    # the pairing matters: half-split and adjacent pairs give different rows
+    a = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv, pairing="half", rotary_dim=rd), None, None)
+    b = ref.qk_prepare_kv_write(qkv, hq, hk, dh, pos, _prep(inv, pairing="adjacent", rotary_dim=rd), None, None)
+    assert not torch.allclose(a.float(), b.float(), atol=1e-2)
 
 
 def test_rotation_angles_are_float32_at_large_positions(ops):
@@ -139,7 +172,7 @@ def test_rotation_angles_are_float32_at_large_positions(ops):
     inv_freq = (1.0 / (10000.0 ** (torch.arange(0, dh, 2).float() / dh))).to(DEV)
     for p in (257, 4099, 131071):
         pos = torch.tensor([p], dtype=torch.int32, device=DEV)
-        q = ops.qk_prepare_kv_write(qkv, 1, 1, dh, pos, inv_freq, None, None, None, None)
+        q = ops.qk_prepare_kv_write(qkv, 1, 1, dh, pos, _prep(inv_freq), None, None)
         assert abs(float(q[0, 0, 0]) - math.cos(float(torch.tensor(float(p)) * inv_freq[0].cpu()))) < 2e-6
         assert abs(float(q[0, 0, 1]) - math.sin(float(torch.tensor(float(p)) * inv_freq[0].cpu()))) < 2e-6
 

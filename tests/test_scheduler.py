@@ -139,3 +139,21 @@ def test_random_loads_always_finish_and_free_everything():
         assert len(done) == 12 and not s.has_work()
         assert all(r.finish_reason in ("length", "out_of_pages") for r in reqs)
         assert cache.num_live() == 0 and all(g.pool.num_held == 0 for g in cache.groups)
+
+
+def test_a_request_ends_at_the_context_limit():
+    cache = _cache(pages=200)
+    s = Scheduler(SchedulerConfig(max_num_batched_tokens=16, decode_batch_size=3, max_seq_len=30), cache)
+    reqs = [Request(0, list(range(25)), SamplingParams(max_decode_length=50)),
+            Request(1, list(range(30)), SamplingParams(max_decode_length=50)),
+            Request(2, list(range(5)), SamplingParams(max_decode_length=4))]
+    for r in reqs:
+        s.add(r)
+    import pytest
+    with pytest.raises(ValueError, match="longer than max_seq_len"):
+        s.add(Request(3, list(range(31))))
+    _drive(s, cache)
+    assert [(len(r.prompt) + len(r.output), r.finish_reason) for r in reqs] == [(30, "length"), (31, "length"),
+                                                                                (9, "length")]
+    assert max(r.num_computed for r in reqs) <= 30  # no token was ever given a position beyond the limit
+    assert cache.num_live() == 0

@@ -90,21 +90,24 @@ def max_live_tokens(steps, round_to=64):
 def run_trace(runner, steps, record_routing=False):
     """Returns ``{rid: logits [T, V]}`` (and ``{rid: {layer: ids [T, k]}}`` if routing is recorded)."""
     rows, routes, done = {}, {}, {}
+    layer_of = {id(b.feed_forward): li for li, b in enumerate(runner.model.blocks)}
     for s in steps:
         entries = [StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]]
         starts = {e.rid: (runner.cache.num_tokens(e.rid) if runner.cache.has_request(e.rid) else 0) for e in entries}
-        logits = runner.step(entries, record_routing=record_routing).float().cpu()
+        seen = {}
+
+        def tap(part, name, value):  # the step's parts hand out what they chose
+            if name == "routing":
+                seen[layer_of[id(part)]] = value[0].clone()
+
+        logits = runner.step(entries, tap=tap if record_routing else None).float().cpu()
         o = t0 = 0
         for e in entries:
             for w in e.want:
                 rows.setdefault(e.rid, {})[starts[e.rid] + w] = logits[o]
                 o += 1
-            if record_routing:
-                for li, b in enumerate(runner.model.blocks):
-                    lr = getattr(b.feed_forward, "last_routing", None)
-                    if lr is not None:
-                        ids = lr[0][t0:t0 + len(e.tokens)].cpu()
-                        routes.setdefault(e.rid, {}).setdefault(li, []).append(ids)
+            for li, ids in seen.items():
+                routes.setdefault(e.rid, {}).setdefault(li, []).append(ids[t0:t0 + len(e.tokens)].cpu())
             t0 += len(e.tokens)
         for rid in s["end"]:
             runner.finish(rid)
