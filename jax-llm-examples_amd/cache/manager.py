@@ -61,6 +61,7 @@ class RequestEntry:
     num_tokens: int = 0  # tokens whose keys and values are written (committed)
     reserved: int = 0  # tokens beyond num_tokens that have pages for the running step
     tables: list[list[int]] = dataclasses.field(default_factory=list)  # per group: page id or -1 per page index
+    versions: list[int] = dataclasses.field(default_factory=list)  # per group: counts the changes of its table
 
 
 @dataclasses.dataclass
@@ -225,7 +226,7 @@ class CacheManager:
         slot = self.slots.alloc()
         for t in self.state.values():
             t[slot].zero_()
-        e = RequestEntry(slot=slot, tables=[[] for _ in self.groups])
+        e = RequestEntry(slot=slot, tables=[[] for _ in self.groups], versions=[0 for _ in self.groups])
         self.requests[rid] = e
         return e
 
@@ -270,6 +271,8 @@ class CacheManager:
         for g, m in zip(self.groups, missing):
             table = e.tables[g.index]
             got = g.pool.alloc(len(m))
+            if got:
+                e.versions[g.index] += 1
             for j, p in zip(m, got):
                 while len(table) <= j:
                     table.append(-1)
@@ -289,6 +292,7 @@ class CacheManager:
             gone = [j for j in range(min(len(table), keep_from // self.page_size)) if table[j] >= 0]
             if gone:
                 self._release(g, [table[j] for j in gone])
+                e.versions[g.index] += 1
                 for j in gone:
                     table[j] = -1
 
@@ -303,6 +307,8 @@ class CacheManager:
             extra = [j for j in range(last_used + 1, len(table)) if table[j] >= 0]
             if extra:
                 self._release(g, [table[j] for j in extra])
+            if len(table) > last_used + 1:
+                e.versions[g.index] += 1
             del table[last_used + 1 :]
 
     def free(self, rid) -> None:
@@ -332,6 +338,10 @@ class CacheManager:
 
     def table(self, rid, group: int) -> list[int]:
         return self.requests[rid].tables[group]
+
+    def table_version(self, rid, group: int) -> int:
+        """Changes whenever the request's block table of this group does (a copy kept elsewhere is then stale)."""
+        return self.requests[rid].versions[group]
 
     def num_free_pages(self) -> list[int]:
         return [g.pool.num_free for g in self.groups]

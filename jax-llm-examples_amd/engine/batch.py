@@ -16,6 +16,13 @@ import numpy as np
 import torch
 
 
+DECODE_BUCKET = 1024
+
+
+def decode_bucket(max_context_len: int) -> int:
+    return -(-max_context_len // DECODE_BUCKET) * DECODE_BUCKET
+
+
 @dataclasses.dataclass
 class StepEntry:
     rid: Any
@@ -32,6 +39,10 @@ class GroupContext:
     seg_lens: list = dataclasses.field(default_factory=list)  # host copies, for kernel work lists
     seg_starts: list = dataclasses.field(default_factory=list)
     meta: dict = dataclasses.field(default_factory=dict)  # kernel launch plans, filled lazily
+    # In a step of single tokens only: the context length the kernels' work is laid out for, a multiple of
+    # DECODE_BUCKET that no request of the step exceeds.  Grids and key ranges then depend on the number of
+    # requests and this bound alone, so a recorded graph of the step fits every step with the same two numbers.
+    decode_bucket: Optional[int] = None
 
 
 @dataclasses.dataclass
@@ -128,7 +139,8 @@ def build_context(ops, dtype, device, cache, entries: Sequence[StepEntry], vocab
         bt = views[7 + 2 * gi].view(R, group_shapes[gi])
         sm = views[8 + 2 * gi]
         groups.append(GroupContext(block_table=bt, slot_mapping=sm, width=group_shapes[gi], retention=g.retention,
-                                   seg_lens=seg_lens, seg_starts=seg_starts))
+                                   seg_lens=seg_lens, seg_starts=seg_starts,
+                                   decode_bucket=decode_bucket(int(ctx_lens.max())) if max(seg_lens) == 1 else None))
     return StepContext(
         ops=ops, dtype=dtype, device=torch.device(device), num_tokens=N, num_segments=R,
         token_ids=token_ids, positions=positions, token_segment=token_segment, cu_seqlens=cu_seqlens,

@@ -1,0 +1,161 @@
+"""The decode fast path: steps that hold one token of every request are recorded once as a
+HIP graph and replayed.
+
+The reference runs its decode steps as one compiled program (``llama4/llama4_jax/model.py:1270-1277``;
+its serving loop scans several decode steps inside one jit, ``serving/serving_jax/serving_loop.py:511-522``).
+Here a step of single tokens is a few hundred kernel launches whose sizes depend on two numbers
+only: how many requests there are, and the bound on their context lengths that the kernels' work
+is laid out for (:func:`~.batch.decode_bucket`).  For each such pair the launches are recorded once;
+everything that changes from step to step (token ids, positions, block tables, slots) lies in one
+persistent device buffer that is refreshed by a single copy before the replay.  Nothing is
+allocated and nothing is cleared with a memset inside a recording.
+
+A recording is made only of models whose parts all say ``graph_safe``; a step that is watched
+(``tap``) runs launch by launch.  Recorded and unrecorded steps launch the same kernels with the
+same arguments, so their logits are equal bit for bit.
+"""
+from __future__ import annotations
+
+import collections
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from .batch import GroupContext, StepContext, StepEntry, decode_bucket
+
+
+class _Recording:
+    """One (number of requests, context bound) pair: its buffers, its context, its graph."""
+
+    def __init__(self, model, cache, ops, num_requests: int, bucket: int) -> None:
+        R, ps = num_requests, cache.page_size
+        dev = model.device
+        self.R, self.bucket = R, bucket
+        self.width = -(-bucket // ps)
+        W = self.width
+        sizes = [("token_ids", R), ("positions", R), ("token_segment", R), ("cu_seqlens", R + 1),
+                 ("context_lens", R), ("state_slots", R), ("logits_indices", R)]
+        for g in cache.groups:
+            sizes += [(f"bt{g.index}", R * W), (f"sm{g.index}", R)]
+        total = sum(n for _, n in sizes)
+        self.mirror = np.zeros(total, np.int32)  # what the device buffer shall hold, kept from step to step
+        self.views, o = {}, 0
+        for name, n in sizes:
+            self.views[name] = (o, o + n)
+            o += n
+        self.host = lambda name: self.mirror[self.views[name][0]: self.views[name][1]]
+        self.host("token_segment")[:] = np.arange(R)
+        self.host("cu_seqlens")[:] = np.arange(R + 1)
+        self.host("logits_indices")[:] = np.arange(R)
+        for g in cache.groups:
+            self.host(f"bt{g.index}")[:] = -1
+        # two pinned staging buffers: the copy of one step may still be on its way when the next is laid out
+        self.staging = [torch.empty(total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.staged = [None, None]  # the event after each buffer's last copy
+        self.turn = 0
+        self.device_buf = torch.zeros(total, dtype=torch.int32, device=dev)
+        d = lambda name: self.device_buf[self.views[name][0]: self.views[name][1]]
+        groups = []
+        for g in cache.groups:
+            groups.append(GroupContext(block_table=d(f"bt{g.index}").view(R, W), slot_mapping=d(f"sm{g.index}"),
+                                       width=W, retention=g.retention, seg_lens=[1] * R, seg_starts=None,
+                                       decode_bucket=bucket))
+        self.ctx = StepContext(
+            ops=ops, dtype=model.dtype, device=dev, num_tokens=R, num_segments=R, token_ids=d("token_ids"),
+            positions=d("positions"), token_segment=d("token_segment"), cu_seqlens=d("cu_seqlens"),
+            context_lens=d("context_lens"), state_slots=d("state_slots"), logits_indices=d("logits_indices"),
+            groups=groups, seg_lens=[1] * R, seg_starts=None, max_seg_len=1, max_context_len=bucket, page_size=ps)
+        self.rows = [None] * R  # per row: (request, its table versions) as last laid out
+        self.graph = None
+        self.logits = None
+
+    def lay_out(self, cache, entries: Sequence[StepEntry], vocab_size: int) -> None:
+        """This step's numbers into the mirror, then one copy to the device."""
+        ps, W = cache.page_size, self.width
+        tok, pos = self.host("token_ids"), self.host("positions")
+        ctx_lens, slots = self.host("context_lens"), self.host("state_slots")
+        for i, e in enumerate(entries):
+            t = int(e.tokens[0])
+            if not 0 <= t < vocab_size:
+                raise ValueError(f"request {e.rid!r}: token id outside 0..{vocab_size - 1}")
+            req = cache.requests[e.rid]
+            p = req.num_tokens
+            tok[i], pos[i], ctx_lens[i], slots[i] = t, p, p + 1, req.slot
+            stamp = (e.rid, tuple(req.versions))
+            fresh = self.rows[i] != stamp
+            for g in cache.groups:
+                table = req.tables[g.index]
+                if fresh:
+                    row = self.host(f"bt{g.index}")[i * W: (i + 1) * W]
+                    row[: len(table)] = table
+                    row[len(table):] = -1
+                page = table[p // ps]
+                if page < 0:
+                    raise AssertionError(f"request {e.rid!r}: a new token has no page in group {g.index}")
+                self.host(f"sm{g.index}")[i] = page * ps + p % ps
+            self.rows[i] = stamp
+        b = self.turn
+        self.turn ^= 1
+        if self.staged[b] is not None:
+            self.staged[b].synchronize()
+        self.staging[b].numpy()[:] = self.mirror
+        self.device_buf.copy_(self.staging[b], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self.staged[b] = ev
+
+
+class DecodeGraphs:
+    MAX_RECORDINGS = 12
+
+    def __init__(self, model, cache, ops) -> None:
+        self.model, self.cache, self.ops = model, cache, ops
+        self.recordings: "collections.OrderedDict[tuple, _Recording]" = collections.OrderedDict()
+        self.pool = None
+        self.replays = 0
+        self.captures = 0
+        self.safe = (getattr(ops, "name", "") == "hip" and model.device.type == "cuda"
+                     and all(getattr(p, "graph_safe", False) for b in model.blocks for p in b.parts().values())
+                     and getattr(model.final_norm, "graph_safe", False))
+
+    def fits(self, entries: Sequence[StepEntry], tap) -> bool:
+        return self.safe and tap is None and all(len(e.tokens) == 1 for e in entries)
+
+    @torch.no_grad()
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """The entries hold reservations for their one token.  Returns float32 logits of the wanted rows; they
+        lie in the recording's own output buffer until the next step of the same shape."""
+        cache, model = self.cache, self.model
+        longest = max(cache.requests[e.rid].num_tokens for e in entries) + 1
+        key = (len(entries), decode_bucket(longest))
+        rec = self.recordings.get(key)
+        if rec is None:
+            rec = _Recording(model, cache, self.ops, *key)
+            self.recordings[key] = rec
+            while len(self.recordings) > self.MAX_RECORDINGS:
+                self.recordings.popitem(last=False)
+        else:
+            self.recordings.move_to_end(key)
+        rec.lay_out(cache, entries, model.plan.vocab_size)
+        if rec.graph is None:
+            # once launch by launch (kernel plans are made, work lists uploaded, libraries warm), then recorded:
+            # a recording runs nothing, and what the step writes (keys, values) it writes again with the same
+            # values when the recording is replayed below
+            model.forward(rec.ctx, cache)
+            torch.cuda.current_stream().synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self.pool):
+                rec.logits = model.forward(rec.ctx, cache)
+            if self.pool is None:
+                self.pool = graph.pool()
+            rec.graph = graph
+            self.captures += 1
+        rec.graph.replay()
+        self.replays += 1
+        wanted = [i for i, e in enumerate(entries) for _ in e.want]
+        if wanted == list(range(len(entries))):
+            return rec.logits
+        if not wanted:
+            return rec.logits[:0]
+        return rec.logits[torch.tensor(wanted, device=rec.logits.device)]

@@ -110,7 +110,7 @@ class Engine:
     def decode_step(self, last_tokens: Sequence[int], ids: Sequence):
         """One token for each live request (``model.py:1270-1277``); returns ``(next_tokens, logits)``."""
         logits = self.runner.step([StepEntry(i, [int(t)], [0]) for i, t in zip(ids, last_tokens)])
-        return self._greedy(logits), logits
+        return self._greedy(logits), logits.clone()  # (the step's own buffer may be written again by the next step)
 
     def _greedy(self, logits) -> list:
         """The largest logit of each row, lowest id among equals (the sampling kernel's greedy case)."""

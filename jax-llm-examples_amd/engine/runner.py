@@ -22,7 +22,17 @@ class ModelRunner:
         self.model = model
         self.cache = cache
         self.ops = ops
-        self.decode_graphs = decode_graphs
+        # steps of single tokens as recorded graphs: on by default where the kernels run and every part allows it
+        self.graphs = None
+        if decode_graphs is None or decode_graphs:
+            from .decode_graph import DecodeGraphs
+
+            graphs = DecodeGraphs(model, cache, ops)
+            if graphs.safe:
+                self.graphs = graphs
+            elif decode_graphs:
+                raise ValueError("decode graphs were asked for, but the kernels do not run here or a part of the "
+                                 "model does not say graph_safe")
         self.steps_run = 0
         self.tokens_run = 0
 
@@ -34,7 +44,9 @@ class ModelRunner:
         after the model has run, the tokens are counted and pages that a
         retention rule has passed are given back.  Returns ``[wanted, vocab]``
         float32, in the order of the entries and of each entry's ``want``.  ``tap``: see
-        :class:`~.batch.StepContext`."""
+        :class:`~.batch.StepContext`.  A step of single tokens may be the replay of a recorded
+        graph (:mod:`.decode_graph`); its logits then lie in that recording's buffer, which the next
+        step of the same shape writes again."""
         cache = self.cache
         seen = set()
         for e in entries:
@@ -56,9 +68,14 @@ class ModelRunner:
                 cache.free(rid)
             raise
         try:
-            ctx = build_context(self.ops, self.model.dtype, self.model.device, cache, entries,
-                                self.model.plan.vocab_size, tap)
-            logits = self.model.forward(ctx, cache)
+            if self.graphs is not None and self.graphs.fits(entries, tap):
+                logits = self.graphs.run(entries)
+                num_tokens = len(entries)
+            else:
+                ctx = build_context(self.ops, self.model.dtype, self.model.device, cache, entries,
+                                    self.model.plan.vocab_size, tap)
+                logits = self.model.forward(ctx, cache)
+                num_tokens = ctx.num_tokens
         except Exception:
             for rid in reserved:
                 cache.cancel(rid)
@@ -68,7 +85,7 @@ class ModelRunner:
         for e in entries:
             cache.commit(e.rid)
         self.steps_run += 1
-        self.tokens_run += ctx.num_tokens
+        self.tokens_run += num_tokens
         return logits
 
     def finish(self, rid) -> None:

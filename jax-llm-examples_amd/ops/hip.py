@@ -360,27 +360,53 @@ class HipOps:
     DECODE_FIT_SPLIT = 1024  # ... at most, to make the items fit in one go
     DECODE_MAX_SPLIT = 512  # ... when there are more items than fit anyway
 
-    def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1, group_size=1):
+    @staticmethod
+    def _most_ranges(retention, bound: int, split: int) -> int:
+        """The most key ranges of ``split`` positions that a query at a position below ``bound`` reads."""
+        kind = retention[0]
+        whole = (bound - 1) // split + 1
+        if kind == "chunk":
+            c = int(retention[1])
+            most = 0
+            for first in range(0, bound, c):
+                last = min(first + c, bound) - 1
+                most = max(most, last // split - first // split + 1)
+            return most
+        if kind == "window":
+            return min(whole, (int(retention[1]) - 1) // split + 2)
+        return whole
+
+    def attention_plan(self, seg_lens, seg_starts, retention, device, num_kv_heads=1, group_size=1, decode_bucket=None):
         """Work lists of the MFMA attention kernels for one step and one retention rule: the rows that are
         single decode tokens (and into how many keys their work is split), tiles of up to 32 consecutive
         tokens of longer segments and, with ``group_size`` > 1 query heads per kv head, the packing of the
-        (tile, head) items of a kv head into blocks of wavefronts that share keys."""
+        (tile, head) items of a kv head into blocks of wavefronts that share keys.  ``decode_bucket``: the step
+        holds single tokens only, none beyond this context length: the split is then chosen from the number of
+        tokens and this bound alone (not from where each request stands), so the same launch fits every such
+        step."""
         from ..parts.base import first_needed_position
 
         dec, tiles, spans, seg_tiles = [], [], [], []
         o = 0
-        for n, start in zip(seg_lens, seg_starts):
+        for i, n in enumerate(seg_lens):
             if n == 1:
                 dec.append(o)
-                spans.append((first_needed_position(retention, start), start))
+                if decode_bucket is None:
+                    spans.append((first_needed_position(retention, seg_starts[i]), seg_starts[i]))
             else:
                 first = len(tiles) // 2
                 for t in range(0, n, self.PREFILL_TILE):
                     tiles += [o + t, min(self.PREFILL_TILE, n - t)]
-                seg_tiles.append((first, len(tiles) // 2 - first, start + n - 1))
+                seg_tiles.append((first, len(tiles) // 2 - first, seg_starts[i] + n - 1))
             o += n
         split, max_splits = self.DECODE_MAX_SPLIT, 1
-        if dec:
+        if dec and decode_bucket is not None:
+            for cand in range(self.DECODE_MIN_SPLIT, self.DECODE_FIT_SPLIT + 1, 32):
+                if num_kv_heads * len(dec) * self._most_ranges(retention, decode_bucket, cand) <= self.DECODE_ITEMS:
+                    split = cand
+                    break
+            max_splits = self._most_ranges(retention, decode_bucket, split)
+        elif dec:
             # the smallest range (a multiple of 32 keys) with which the work items still fit the GPU in one go:
             # a compute unit that gets a second item beside its first takes much longer than the others
             for cand in range(self.DECODE_MIN_SPLIT, self.DECODE_FIT_SPLIT + 1, 32):
@@ -436,7 +462,8 @@ class HipOps:
                             seg_lens.append(0)
                             seg_starts.append(pos[i])
                         seg_lens[-1] += 1
-                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk, hq // hk)
+                plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk, hq // hk,
+                                           decode_bucket=meta.decode_bucket if meta is not None else None)
                 if meta is not None:
                     meta.meta[key] = plan
             if plan["num_tiles"]:
@@ -461,7 +488,9 @@ class HipOps:
         splits, tiles_per_split, ws_ml, ws_o = 1, 0, None, None
         waves = n * hq
         if waves < self.GENERIC_SPLIT_BELOW:
-            if meta is not None:
+            if meta is not None and meta.decode_bucket is not None:
+                longest = meta.decode_bucket  # (a step of single tokens: laid out for the bound, see GroupContext)
+            elif meta is not None:
                 longest = max(s0 + ln for s0, ln in zip(meta.seg_starts, meta.seg_lens))
             else:
                 longest = int(positions.max()) + 1

@@ -28,13 +28,19 @@ def _vocab(name):
     return c.get("text_config", c)["vocab_size"]
 
 
-def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu"):
+def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu", record=True):
+    """``record``: watch every step for the experts it chose (a watched step is never the replay of a recorded
+    graph); without it, steps of single tokens go through the recorded decode graphs."""
     lengths = LENGTHS[name] + (LENGTHS[name][::-1] + LENGTHS[name] if mode == "mixed" else [])
     reqs = traces.random_requests(_vocab(name), lengths, seed=5)
     steps = MODES[mode](reqs)
     runner = make_runner(folder, dtype, traces.max_live_tokens(steps), device, reference_ops=reference_ops,
                          poison=True)
-    got, routes = traces.run_trace(runner, steps, record_routing=True)
+    if record:
+        got, routes = traces.run_trace(runner, steps, record_routing=True)
+    else:
+        got, routes = traces.run_trace(runner, steps), {}
+        assert runner.graphs is not None and runner.graphs.replays > 0 and runner.graphs.captures > 0
     if mode == "mixed":  # so few pages that they were used again
         assert all(g.pool.handed_out > g.pool.num_pages for g in runner.cache.groups)
     runner.cache.check()
@@ -80,6 +86,41 @@ def test_cpu_plain_ops_float32(model_dirs, name, mode):
 @pytest.mark.parametrize("name", list(TINY))
 def test_gpu_float32(model_dirs, name, mode):
     _check(name, model_dirs[name], "float32", "cuda:0", mode, reference_ops=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["tail", "mixed"])
+@pytest.mark.parametrize("name", list(TINY))
+def test_gpu_float32_with_recorded_decode_steps(model_dirs, name, mode):
+    """The same comparison with the steps of single tokens replayed from recorded HIP graphs."""
+    _check(name, model_dirs[name], "float32", "cuda:0", mode, reference_ops=False, record=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "F"])
+def test_recorded_decode_steps_equal_unrecorded_ones_bit_for_bit(model_dirs, model_dirs_bf16, tmp_path, name, dtype):
+    """Replays and launch-by-launch steps run the same kernels with the same arguments.  Between the replays lie
+    the trace's other steps (portions of prompts, launch by launch) and a synchronisation after every step."""
+    if name == "F":
+        folder = write_tiny("F", str(tmp_path / "F"), torch.bfloat16)
+    else:
+        folder = (model_dirs if dtype == "float32" else model_dirs_bf16)[name]
+    lengths = LENGTHS[name]
+    reqs = traces.random_requests(_vocab(name), lengths + lengths[::-1], seed=8)
+    for mode in ("tail", "mixed"):
+        steps = MODES[mode](reqs)
+        out = {}
+        for graphs in (False, True):
+            runner = make_runner(folder, dtype, traces.max_live_tokens(steps), "cuda:0", poison=True,
+                                 decode_graphs=graphs)
+            out[graphs] = traces.run_trace(runner, steps)
+            if graphs:
+                assert runner.graphs.replays > 20 and 0 < runner.graphs.captures < runner.graphs.replays
+            else:
+                assert runner.graphs is None
+        for rid in reqs:
+            assert torch.equal(out[True][rid], out[False][rid]), (mode, rid)
 
 
 @pytest.mark.gpu
