@@ -196,11 +196,29 @@ __device__ __forceinline__ V load_kv(const void* p) {
   return ONCE ? __builtin_nontemporal_load(reinterpret_cast<const V*>(p)) : *reinterpret_cast<const V*>(p);
 }
 
+// The queries of the wavefront's columns as B operands of the first product (zeros for columns without keys).
+template <int DH, int CT>
+__device__ __forceinline__ void load_queries(const bf16_t* __restrict__ q, const Columns (&col)[CT], int Hq,
+                                             bf16x8 (&qb)[CT][DH / 32]) {
+  const int g = (threadIdx.x & 63) >> 4;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const bf16_t* qrow = q + ((size_t)col[ct].token * Hq + col[ct].head) * DH + g * 8;
+    const bool ok = col[ct].lo <= col[ct].hi;
+#pragma unroll
+    for (int c = 0; c < DH / 32; ++c) {
+      uint4 v = {0u, 0u, 0u, 0u};
+      if (ok) v = *reinterpret_cast<const uint4*>(qrow + c * 32);
+      qb[ct][c] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+}
+
 template <int DH, int CT, bool ONCE>
-__device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv,
-                                       const int* __restrict__ table, const Columns (&col)[CT], int k_lo, int k_hi,
-                                       int hk, int Hq, int Hkv, int ps, float scale_log2, float (&m)[CT],
-                                       float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad) {
+__device__ __forceinline__ void attend_with(const bf16x8 (&qb)[CT][DH / 32], const bf16_t* __restrict__ kv,
+                                            const int* __restrict__ table, const Columns (&col)[CT], int k_lo,
+                                            int k_hi, int hk, int Hkv, int ps, float scale_log2, float (&m)[CT],
+                                            float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad) {
   const int lane = threadIdx.x & 63;
   const int c16 = lane & 15, g = lane >> 4;
   constexpr int KC = DH / 32;  // k-steps of the first product
@@ -208,17 +226,8 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
   const size_t plane = (size_t)ps * DH;
   const size_t page_stride = 2 * (size_t)Hkv * plane;
 
-  bf16x8 qb[CT][KC];
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
-    const bf16_t* qrow = q + ((size_t)col[ct].token * Hq + col[ct].head) * DH + g * 8;
-    const bool ok = col[ct].lo <= col[ct].hi;
-#pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      uint4 v = {0u, 0u, 0u, 0u};
-      if (ok) v = *reinterpret_cast<const uint4*>(qrow + c * 32);
-      qb[ct][c] = __builtin_bit_cast(bf16x8, v);
-    }
     m[ct] = -INFINITY;
     l[ct] = 0.f;
 #pragma unroll
@@ -322,6 +331,16 @@ __device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_
   }
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) l[ct] = column_sum(l[ct]);
+}
+
+template <int DH, int CT, bool ONCE>
+__device__ __forceinline__ void attend(const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv,
+                                       const int* __restrict__ table, const Columns (&col)[CT], int k_lo, int k_hi,
+                                       int hk, int Hq, int Hkv, int ps, float scale_log2, float (&m)[CT],
+                                       float (&l)[CT], f32x4 (&acc)[CT][DH / 16], bool& bad) {
+  bf16x8 qb[CT][DH / 32];
+  load_queries<DH, CT>(q, col, Hq, qb);
+  attend_with<DH, CT, ONCE>(qb, kv, table, col, k_lo, k_hi, hk, Hkv, ps, scale_log2, m, l, acc, bad);
 }
 
 // ------------------------------------------------------------------ prefill portions
@@ -733,6 +752,277 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ ws_ml, c
   }
 }
 
+// ------------------------------------------------------------------ decode, from the projection's rows
+// The decode kernel above with what comes before and after it folded in, for steps of single tokens.  A block is
+// four wavefronts that take four consecutive key ranges of one (token, kv head):
+//   * the sines and cosines of the token's position are formed once per block;
+//   * a wavefront takes its queries straight from the fused q|k|v rows and prepares them itself (rotation by
+//     adjacent pairs, weightless rms norm over the head, position-dependent scale: see attention_prep.hip);
+//   * the wavefront whose range holds the token's own position prepares that token's key, writes key and value
+//     into their page and then reads them back with the rest of its range;
+//   * the block's four partial results are merged in shared memory; if the token has no more than four ranges
+//     that is the output; otherwise the block's result is written through to where all dies see it, and the
+//     block of the (token, kv head) that finishes last merges the blocks' results and writes the output rows.
+// `tickets` holds one counter per (decode token, kv head); they are zero between launches (the merging block puts
+// its counter back), so the buffer is cleared once, when it is made.  max_splits is a multiple of 4.
+//   qkv: [N][(Hq + 2 Hkv) * DH]; inv_freq: [DH / 2] or null; norm_eps < 0: no norm; floor_scale <= 0: no scale
+//   ws_ml: [(d * Hkv + hk) * (max_splits / 4) + block][G][2], ws_o: the same with [G][DH]
+// dynamic shared memory: DH floats (sines, cosines) + 4 * G * (DH + 2) floats (the wavefronts' results)
+
+// A float written to / read from where all compute units of the GPU see it at once (the caches of one die are
+// written through and read past): for data that blocks on different dies hand each other within a launch.
+__device__ __forceinline__ void put_shared(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float get_shared(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+struct PrepArgs {
+  const float* inv_freq;
+  float norm_eps, floor_scale, attn_scale;
+  const int* slot_mapping;
+  int write_kv;
+};
+
+constexpr int kFusedWaves = 4;
+
+template <int DH, int CT>
+__global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention_decode_fused_kernel(
+    const bf16_t* __restrict__ qkv, bf16_t* __restrict__ kv, bf16_t* __restrict__ out, float* __restrict__ ws_ml,
+    float* __restrict__ ws_o, int* __restrict__ tickets, const int* __restrict__ positions,
+    const int* __restrict__ token_segment, const int* __restrict__ block_table, int table_width,
+    const int* __restrict__ dec_tokens, int num_dec, int max_splits, int kSplit, int ret_mode, int ret_param,
+    float scale_log2, int Hq, int Hkv, int ps, PrepArgs prep) {
+  constexpr int KC = DH / 32;
+  extern __shared__ float smem[];
+  __shared__ int last_flag;
+  const int G = Hq / Hkv;
+  float* sincos = smem;                     // [DH / 2][2]
+  float* part_ml = smem + DH;               // [4][G][2]
+  float* part_o = part_ml + kFusedWaves * G * 2;  // [4][G][DH]
+  const int lane = threadIdx.x & 63, wave = wave_index();
+  const int blocks_per = max_splits / kFusedWaves;
+  const int bsplit = blockIdx.x % blocks_per;
+  const int hk = (blockIdx.x / blocks_per) % Hkv;
+  const int d = blockIdx.x / (blocks_per * Hkv);
+  const int n = dec_tokens[d];
+  const int pos = positions[n];
+  const int first = first_key(ret_mode, ret_param, pos);
+  const int num_ranges = pos / kSplit - first / kSplit + 1;
+  if (bsplit * kFusedWaves >= num_ranges) return;  // (the whole block: this token has fewer ranges)
+  const int num_blocks = (num_ranges + kFusedWaves - 1) / kFusedWaves;
+  const int split = bsplit * kFusedWaves + wave;
+  const bool active = split < num_ranges;
+  const int s_abs = first / kSplit + split;
+  const int k_lo = max(first, s_abs * kSplit), k_hi = min(pos, s_abs * kSplit + kSplit - 1);
+  const int c16 = lane & 15, g = lane >> 4;
+  const bf16_t* row = qkv + (size_t)n * (Hq + 2 * Hkv) * DH;
+  const int* table = block_table + (size_t)token_segment[n] * table_width;
+
+  if (prep.inv_freq != nullptr) {
+    for (int j = threadIdx.x; j < DH / 2; j += blockDim.x) {
+      const float ang = (float)pos * prep.inv_freq[j];
+      sincos[2 * j] = sinf(ang);
+      sincos[2 * j + 1] = cosf(ang);
+    }
+    __syncthreads();
+  }
+
+  float m[CT], l[CT];
+  f32x4 acc[CT][DH / 16];
+  bool bad = false;
+  if (active) {
+    // ---- this token's key and value go into their page (by the wavefront that will read them)
+    if (prep.write_kv && k_hi == pos) {
+      const int slot = prep.slot_mapping[n];
+      const int page = slot / ps, off = slot - page * ps;
+      const size_t plane = (size_t)ps * DH;
+      bf16_t* kplane = kv + ((size_t)page * 2 * Hkv + hk) * plane;
+      bf16_t* vplane = kplane + (size_t)Hkv * plane;
+      const bf16_t* ksrc = row + (size_t)(Hq + hk) * DH;
+      const bf16_t* vsrc = row + (size_t)(Hq + Hkv + hk) * DH;
+      constexpr int PPL = (DH / 2 + 63) / 64;  // pairs per lane
+      float ka[PPL], kb2[PPL];
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < PPL; ++i) {
+        const int j = lane + 64 * i;
+        ka[i] = 0.f;
+        kb2[i] = 0.f;
+        if (j < DH / 2) {
+          const uint32_t w = *reinterpret_cast<const uint32_t*>(ksrc + 2 * j);
+          float x1 = __uint_as_float(w << 16), x2 = __uint_as_float(w & 0xffff0000u);
+          if (prep.inv_freq != nullptr) {
+            const float sn = sincos[2 * j], cs = sincos[2 * j + 1];
+            const float r1 = x1 * cs - x2 * sn, r2 = x2 * cs + x1 * sn;
+            x1 = r1;
+            x2 = r2;
+          }
+          ka[i] = x1;
+          kb2[i] = x2;
+          ss += x1 * x1 + x2 * x2;
+        }
+      }
+      float mul = 1.f;
+      if (prep.norm_eps >= 0.f) mul = 1.0f / sqrtf(wave_sum(ss) / (float)DH + prep.norm_eps);
+#pragma unroll
+      for (int i = 0; i < PPL; ++i) {
+        const int j = lane + 64 * i;
+        if (j < DH / 2) {
+          *reinterpret_cast<uint32_t*>(kplane + (size_t)off * DH + 2 * j) = pack_bf16(ka[i] * mul, kb2[i] * mul);
+          const uint32_t w = *reinterpret_cast<const uint32_t*>(vsrc + 2 * j);
+          vplane[(size_t)(2 * j) * ps + off] = (bf16_t)(w & 0xffffu);
+          vplane[(size_t)(2 * j + 1) * ps + off] = (bf16_t)(w >> 16);
+        }
+      }
+      // what the lanes wrote is read back by other lanes of this wavefront below
+      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+    }
+
+    // ---- the queries of this kv head's group, prepared in registers
+    Columns col[CT];
+    bf16x8 qb[CT][KC];
+    float q_mul = 1.f;
+    if (prep.floor_scale > 0.f)
+      q_mul = 1.0f + prep.attn_scale * log1pf(floorf(((float)pos + 1.0f) / prep.floor_scale));
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const int c = ct * 16 + c16;
+      const bool ok = c < G;
+      col[ct].token = n;
+      col[ct].head = ok ? hk * G + c : hk * G;
+      col[ct].lo = ok ? k_lo : 1;
+      col[ct].hi = ok ? k_hi : 0;
+      const bf16_t* qrow = row + (size_t)col[ct].head * DH + g * 8;
+      float x[KC][8];
+      float ss = 0.f;
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc) {
+        const uint4 r = *reinterpret_cast<const uint4*>(qrow + kc * 32);
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float x1 = __uint_as_float(w[i] << 16), x2 = __uint_as_float(w[i] & 0xffff0000u);
+          if (prep.inv_freq != nullptr) {
+            const int j = kc * 16 + g * 4 + i;
+            const float sn = sincos[2 * j], cs = sincos[2 * j + 1];
+            const float r1 = x1 * cs - x2 * sn, r2 = x2 * cs + x1 * sn;
+            x1 = r1;
+            x2 = r2;
+          }
+          x[kc][2 * i] = x1;
+          x[kc][2 * i + 1] = x2;
+          ss += x1 * x1 + x2 * x2;
+        }
+      }
+      float mul = q_mul;
+      if (prep.norm_eps >= 0.f) mul = (1.0f / sqrtf(column_sum(ss) / (float)DH + prep.norm_eps)) * q_mul;
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc) {
+        uint4 v = {0u, 0u, 0u, 0u};
+        if (ok)
+          v = uint4{pack_bf16(x[kc][0] * mul, x[kc][1] * mul), pack_bf16(x[kc][2] * mul, x[kc][3] * mul),
+                    pack_bf16(x[kc][4] * mul, x[kc][5] * mul), pack_bf16(x[kc][6] * mul, x[kc][7] * mul)};
+        qb[ct][kc] = __builtin_bit_cast(bf16x8, v);
+      }
+    }
+    attend_with<DH, CT, true>(qb, kv, table, col, k_lo, k_hi, hk, Hkv, ps, scale_log2, m, l, acc, bad);
+    bad = __any(bad);
+  }
+
+  // ---- the block's wavefronts hand their results to each other
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = ct * 16 + c16;
+    if (c >= G) continue;
+    if (g == 0) {
+      part_ml[(wave * G + c) * 2] = !active ? -INFINITY : (bad ? __builtin_nanf("") : m[ct]);
+      part_ml[(wave * G + c) * 2 + 1] = active ? l[ct] : 0.f;
+    }
+    if (active) {
+      float* o = part_o + ((size_t)wave * G + c) * DH + 4 * g;
+#pragma unroll
+      for (int dt = 0; dt < DH / 16; ++dt) *reinterpret_cast<f32x4*>(o + dt * 16) = acc[ct][dt];
+    }
+  }
+  __syncthreads();
+  const bool alone = num_blocks == 1;
+  const size_t unit = ((size_t)d * Hkv + hk) * blocks_per;  // this (token, kv head)'s first block result
+  for (int idx = threadIdx.x; idx < G * DH; idx += blockDim.x) {
+    const int c = idx / DH, e = idx - c * DH;
+    float mx = -INFINITY;
+    bool nan = false;
+#pragma unroll
+    for (int w = 0; w < kFusedWaves; ++w) {
+      const float ms = part_ml[(w * G + c) * 2];
+      nan = nan || ms != ms;
+      mx = fmaxf(mx, ms);
+    }
+    float lsum = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < kFusedWaves; ++w) {
+      const float ms = part_ml[(w * G + c) * 2];
+      const bool use = ms != -INFINITY && ms == ms;
+      const float f = use ? exp2f(ms - mx) : 0.f;
+      lsum += use ? part_ml[(w * G + c) * 2 + 1] * f : 0.f;
+      o += use ? part_o[((size_t)w * G + c) * DH + e] * f : 0.f;
+    }
+    if (alone) {
+      const float r = nan ? __builtin_nanf("") : (lsum > 0.f ? o / lsum : 0.f);
+      out[((size_t)n * Hq + hk * G + c) * DH + e] = float_to_bf16(r);
+    } else {
+      put_shared(ws_o + ((unit + bsplit) * G + c) * DH + e, o);
+      if (e == 0) {
+        put_shared(ws_ml + ((unit + bsplit) * G + c) * 2, nan ? __builtin_nanf("") : mx);
+        put_shared(ws_ml + ((unit + bsplit) * G + c) * 2 + 1, lsum);
+      }
+    }
+  }
+  if (alone) return;
+
+  // ---- the last of the (token, kv head)'s blocks to get here merges the blocks' results
+  // They were written through to where every compute unit reads them (put_shared); once a thread's writes are
+  // done (the fence waits for them) and all threads have got there (the barrier), the ticket is taken, and the
+  // block that takes the last one reads the results from that same place (get_shared), not from a cache of its
+  // own die.  No cache is written back or emptied as a whole, as a fence over the whole GPU would do.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int ticket = __hip_atomic_fetch_add(&tickets[d * Hkv + hk], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last_flag = ticket == num_blocks - 1;
+    if (last_flag) __hip_atomic_store(&tickets[d * Hkv + hk], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!last_flag) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  for (int idx = threadIdx.x; idx < G * DH; idx += blockDim.x) {
+    const int c = idx / DH, e = idx - c * DH;
+    const float* ml = ws_ml + (unit * G + c) * 2;  // block b: + b * G * 2
+    const float* wo = ws_o + (unit * G + c) * DH + e;  // block b: + b * G * DH
+    float mx = -INFINITY;
+    bool nan = false;
+    for (int b = 0; b < num_blocks; ++b) {
+      const float ms = get_shared(ml + (size_t)b * G * 2);
+      nan = nan || ms != ms;
+      mx = fmaxf(mx, ms);
+    }
+    float lsum = 0.f, o = 0.f;
+#pragma unroll 8
+    for (int b = 0; b < num_blocks; ++b) {
+      const float ms = get_shared(ml + (size_t)b * G * 2);
+      const float ls = get_shared(ml + (size_t)b * G * 2 + 1);
+      const float v = get_shared(wo + (size_t)b * G * DH);
+      const bool use = ms != -INFINITY && ms == ms;
+      const float f = use ? exp2f(ms - mx) : 0.f;
+      lsum += use ? ls * f : 0.f;
+      o += use ? v * f : 0.f;
+    }
+    const float r = nan ? __builtin_nanf("") : (lsum > 0.f ? o / lsum : 0.f);
+    out[((size_t)n * Hq + hk * G + c) * DH + e] = float_to_bf16(r);
+  }
+}
+
 static bool head_dim_ok(int dh) { return dh == 32 || dh == 64 || dh == 96 || dh == 128 || dh == 256; }
 
 // Wavefronts, and so (tile, head) items, per block of the key-sharing prefill kernel: one per SIMD, and two
@@ -837,6 +1127,52 @@ JLE_API int jle_attention_decode(const void* q, const void* kv, void* out, float
   JLE_LAUNCH_CHECK();
   hipLaunchKernelGGL(attention_decode_merge_kernel, dim3(num_dec * Hq), dim3(dh <= 64 ? 64 : 128), 0, s, ws_ml, ws_o,
                      (bf16_t*)out, positions, dec_tokens, max_splits, split, ret_mode, ret_param, Hq, Hkv, dh, 16 * ct);
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
+// Steps of single tokens: queries, the new key and value, attention and the merge of the key ranges in one launch
+// (see attention_decode_fused_kernel).  tickets: num_dec * Hkv counters, zero before the first launch and after
+// every launch.  max_splits: a multiple of 4.  ws_ml needs num_dec * Hkv * (max_splits / 4) * G * 2 floats, ws_o
+// that many * dh / 2, G = Hq / Hkv.
+JLE_API int jle_attention_decode_fused(const void* qkv, void* kv, void* out, float* ws_ml, float* ws_o, int* tickets,
+                                       const int* positions, const int* token_segment, const int* block_table,
+                                       int table_width, const int* dec_tokens, int num_dec, int max_splits, int split,
+                                       int ret_mode, int ret_param, float scale, int Hq, int Hkv, int dh, int ps,
+                                       const float* inv_freq, float norm_eps, float floor_scale, float attn_scale,
+                                       const int* slot_mapping, int write_kv, hipStream_t s) {
+  if (num_dec <= 0) return 0;
+  if (!jle_attention_mfma_supported(dh, Hq, Hkv, ps) || max_splits < 1 || split < 32 || split % 32) return JLE_BAD_ARG;
+  if ((ret_mode == 1 || ret_mode == 2) && ret_param <= 0) return JLE_BAD_ARG;
+  if (tickets == nullptr || (write_kv && slot_mapping == nullptr) || max_splits % kFusedWaves) return JLE_BAD_ARG;
+  const int G = Hq / Hkv;
+  if (G > 32) return JLE_BAD_ARG;
+  const int ct = G > 16 ? 2 : 1;
+  const size_t lds = ((size_t)dh + (size_t)kFusedWaves * G * (dh + 2)) * sizeof(float);
+  if (lds > 48 * 1024) return JLE_BAD_ARG;
+  const long long blocks = (long long)num_dec * Hkv * (max_splits / kFusedWaves);
+  if (blocks > 0x7fffffffll) return JLE_BAD_ARG;
+  dim3 g((unsigned)blocks), b(64 * kFusedWaves);
+  const float sl = scale * kLog2e;
+  const PrepArgs prep = {inv_freq, norm_eps, floor_scale, attn_scale, slot_mapping, write_kv};
+#define LAUNCH(DH, CT)                                                                                            \
+  hipLaunchKernelGGL((attention_decode_fused_kernel<DH, CT>), g, b, lds, s, (const bf16_t*)qkv, (bf16_t*)kv,       \
+                     (bf16_t*)out, ws_ml, ws_o, tickets, positions, token_segment, block_table, table_width,      \
+                     dec_tokens, num_dec, max_splits, split, ret_mode, ret_param, sl, Hq, Hkv, ps, prep)
+#define PICK(DH)                \
+  do {                          \
+    if (ct == 1) LAUNCH(DH, 1); \
+    else LAUNCH(DH, 2);         \
+  } while (0)
+  switch (dh) {
+    case 32: PICK(32); break;
+    case 64: PICK(64); break;
+    case 96: PICK(96); break;
+    case 128: PICK(128); break;
+    case 256: PICK(256); break;
+  }
+#undef PICK
+#undef LAUNCH
   JLE_LAUNCH_CHECK();
   return 0;
 }

@@ -37,6 +37,8 @@ _SIGNATURES = {
     "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
     "jle_attention_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i,
                              _vp],
+    "jle_attention_decode_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i,
+                                   _i, _i, _vp, _f, _f, _f, _vp, _i, _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
@@ -98,6 +100,9 @@ class HipOps:
         raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         self._raw_stream = raw if raw is not None else (lambda i: torch.cuda.current_stream(i).cuda_stream)
         # true float32 products: no reduced-precision matrix mode
+        # counters of the kernels in which the last wavefront (or block) to finish does the closing work: zero
+        # between launches (whoever closes puts its counter back), so they are cleared here once
+        self._tickets = torch.zeros(self.TICKETS, dtype=torch.int32, device=self.device)
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
         torch.set_float32_matmul_precision("highest")
@@ -352,6 +357,53 @@ class HipOps:
                    n, hq, hk, dh, max(ps, 1), 0 if kv_cache is None else 1, pairing, rd, _p(prep.norm_weight_q),
                    _p(prep.norm_weight_k), int(bool(prep.norm_first)))
         return q
+
+    TICKETS = 1 << 16
+
+    def attention_from_qkv(self, qkv, num_heads, num_kv_heads, head_dim, positions, token_segment, prep, kv_cache,
+                           writes: bool, slot_mapping, block_table, retention, scale: float, meta=None):
+        """From the fused q|k|v rows to the attention output ``[N, num_heads * head_dim]``: q and k prepared as
+        ``prep`` says, k and v written into their pages (if this run ``writes`` its cache), attention over the
+        pages.  A step of single tokens in bfloat16 is one launch (``attention_decode_fused_kernel``)."""
+        n = qkv.shape[0]
+        hq, hk, dh = num_heads, num_kv_heads, head_dim
+        ps = kv_cache.shape[3]
+        group = hq // max(hk, 1)
+        if (meta is not None and meta.decode_bucket is not None and qkv.dtype == torch.bfloat16 and prep.plain
+                and group <= 32 and n * hk <= self.TICKETS and 4 * (dh + 4 * group * (dh + 2)) <= 48 * 1024
+                and self.lib.jle_attention_mfma_supported(dh, hq, hk, ps)):
+            self._chk(qkv, kv_cache.dtype, (n, (hq + 2 * hk) * dh), "q|k|v")
+            self._chk(kv_cache, None, (kv_cache.shape[0], 2, hk, ps, dh), "kv pages")
+            self._chk(block_table, torch.int32, None, "block table")
+            self._chk(positions, torch.int32, (n,), "positions")
+            self._chk(token_segment, torch.int32, (n,), "token segments")
+            if writes:
+                self._chk(slot_mapping, torch.int32, (n,), "slot mapping")
+            inv_freq = None if prep.rotation is None else prep.rotation.inv_freq
+            if inv_freq is not None:
+                self._chk(inv_freq, torch.float32, (dh // 2,), "inv_freq")
+            key = f"attn_plan_{hq // hk}"
+            plan = meta.meta.get(key)
+            if plan is None:
+                plan = self.attention_plan(meta.seg_lens, meta.seg_starts, retention, qkv.device, hk, hq // hk,
+                                           decode_bucket=meta.decode_bucket)
+                meta.meta[key] = plan
+            splits = -(-plan["max_splits"] // 4) * 4  # a block takes four ranges
+            units = n * hk * (splits // 4) * group
+            ws_ml = torch.empty(units * 2, dtype=torch.float32, device=qkv.device)
+            ws_o = torch.empty(units * dh, dtype=torch.float32, device=qkv.device)
+            out = torch.empty(n, hq * dh, dtype=qkv.dtype, device=qkv.device)
+            fs, sc = (prep.query_scale if prep.query_scale is not None else (0.0, 0.0))
+            mode = _RET_MODES[retention[0]]
+            param = int(retention[1]) if len(retention) > 1 else 0
+            self._call("jle_attention_decode_fused", _p(qkv), _p(kv_cache), _p(out), _p(ws_ml), _p(ws_o),
+                       _p(self._tickets), _p(positions), _p(token_segment), _p(block_table), block_table.shape[1],
+                       _p(plan["dec"]), n, splits, plan["split"], mode, param, float(scale), hq, hk, dh,
+                       ps, _p(inv_freq), -1.0 if prep.norm_eps is None else float(prep.norm_eps), float(fs),
+                       float(sc), _p(slot_mapping) if writes else None, int(bool(writes)))
+            return out
+        q = self.qk_prepare_kv_write(qkv, hq, hk, dh, positions, prep, kv_cache if writes else None, slot_mapping)
+        return self.paged_attention(q, kv_cache, block_table, positions, token_segment, retention, scale, meta)
 
     PREFILL_TILE = 32  # tokens per prefill work item (the kernels take 16 or 32)
     GENERIC_SPLIT_BELOW = 2048  # the float32-arithmetic attention: fewer (token, head) pairs than this share their keys

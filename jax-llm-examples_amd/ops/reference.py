@@ -136,6 +136,13 @@ class ReferenceOps:
             values_t(kv_cache)[page, :, :, off] = v.to(kv_cache.dtype)
         return q.to(dt)
 
+    def attention_from_qkv(self, qkv, num_heads, num_kv_heads, head_dim, positions, token_segment, prep, kv_cache,
+                           writes: bool, slot_mapping, block_table, retention, scale: float, meta=None):
+        """q and k prepared, k and v written (if this run writes its cache), attention over the pages."""
+        q = self.qk_prepare_kv_write(qkv, num_heads, num_kv_heads, head_dim, positions, prep,
+                                     kv_cache if writes else None, slot_mapping)
+        return self.paged_attention(q, kv_cache, block_table, positions, token_segment, retention, scale, meta)
+
     def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
         """For each token: softmax over the keys of its own request at positions
         ``[start(pos), pos]``, read from the pages its block table names."""

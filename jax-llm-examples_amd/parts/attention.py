@@ -73,18 +73,9 @@ class Attention(Mixer):
     def forward(self, h: torch.Tensor, ctx, cache) -> torch.Tensor:
         ops = ctx.ops
         qkv = ops.linear(h, self.params["wqkv"])
-        q = ops.qk_prepare_kv_write(
-            qkv,
-            self.num_heads,
-            self.num_kv_heads,
-            self.head_dim,
-            ctx.positions,
-            self.prep,
-            cache.kv if cache.writes else None,
-            cache.slot_mapping,
-        )
-        o = ops.paged_attention(
-            q, cache.kv, cache.block_table, ctx.positions, ctx.token_segment, self.retention,
-            self.softmax_scale, cache.attn_meta,
+        o = ops.attention_from_qkv(
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim, ctx.positions, ctx.token_segment, self.prep,
+            cache.kv, cache.writes, cache.slot_mapping, cache.block_table, self.retention, self.softmax_scale,
+            cache.attn_meta,
         )
         return ops.linear(o, self.params["wo"])

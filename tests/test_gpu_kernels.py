@@ -210,6 +210,93 @@ def test_paged_attention(ops, ref, dt, hq, hk, dh, ps, retention):
     _assert_close_to_scale(got, want, dt)
 
 
+def _decode_case(hq, hk, dh, ps, dt, contexts, seed=0):
+    """One new token per request after ``contexts[i]`` tokens in the cache; the step's group context with the
+    bound the kernels' work is laid out for; raw q|k|v rows and the slots of the new tokens."""
+    from jax_llm_examples_amd.engine.batch import GroupContext, decode_bucket
+    q, kv, bt, pos, seg = _attention_case(hq, hk, dh, ps, dt, [(c, 1) for c in contexts], seed=seed)
+    n = len(contexts)
+    g = torch.Generator().manual_seed(seed + 50)
+    qkv = torch.randn(n, (hq + 2 * hk) * dh, generator=g).to(dt).to(DEV)
+    slots = torch.tensor([int(bt[i, c // ps]) * ps + c % ps for i, c in enumerate(contexts)], dtype=torch.int32,
+                         device=DEV)
+    meta = lambda ret: GroupContext(block_table=bt, slot_mapping=slots, width=bt.shape[1], retention=ret,
+                                    seg_lens=[1] * n, seg_starts=list(contexts),
+                                    decode_bucket=decode_bucket(max(contexts) + 1))
+    return qkv, kv, bt, pos, seg, slots, meta
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("hq,hk,dh,ps,contexts", [
+    (40, 8, 128, 16, [3000 + 94 * i for i in range(64)]),  # the serving shape: 64 requests between 3,000 and 9,000
+    (40, 8, 128, 16, [8191, 8192, 8193, 0, 5, 16383, 16384, 4095]),
+    (10, 2, 64, 32, [0, 1, 31, 32, 700, 129]), (6, 1, 32, 16, [77]), (20, 1, 96, 48, [500, 47, 48]),
+    (34, 2, 32, 16, [260, 3]), (4, 4, 256, 16, [90, 1000])])
+@pytest.mark.parametrize("retention", [("all",), ("chunk", 8192), ("chunk", 96), ("window", 200)])
+def test_attention_of_a_step_of_single_tokens_from_the_projection_rows(ops, ref, dt, hq, hk, dh, ps, contexts, retention):
+    """Rotation, q/k norm, scale, the write of the new key and value, attention over many key ranges and their
+    merge: one launch in bfloat16 (two kernels and a merge in float32), against the plain ops."""
+    if retention == ("chunk", 8192) and max(contexts) < 3000:
+        pytest.skip("the large chunk is for the long contexts")
+    from jax_llm_examples_amd.ops.hip import HipOps
+    qkv, kv, bt, pos, seg, slots, meta = _decode_case(hq, hk, dh, ps, dt, contexts)
+    inv = (1.0 / (10000.0 ** (torch.arange(0, dh, 2).float() / dh))).to(DEV)
+    for prep in (_prep(inv, 1e-5, None), _prep(None, None, (64.0, 0.2)), _prep(inv, None, None)):
+        kv1, kv2 = kv.clone(), kv.clone()
+        calls = []
+        inner = ops._call
+        ops._call = lambda name, *a: (calls.append(name), inner(name, *a))[1]
+        try:
+            got = ops.attention_from_qkv(qkv, hq, hk, dh, pos, seg, prep, kv1, True, slots, bt, retention,
+                                         dh ** -0.5, meta(retention))
+        finally:
+            ops._call = inner
+        if dt == torch.bfloat16:
+            assert calls == ["jle_attention_decode_fused"], calls
+        want = ref.attention_from_qkv(qkv, hq, hk, dh, pos, seg, prep, kv2, True, slots, bt, retention, dh ** -0.5)
+        _assert_close_to_scale(got, want, dt)
+        assert torch.allclose(kv1.float(), kv2.float(), **_tol(dt))  # the new keys and values are in their pages
+        assert int(ops._tickets.abs().sum()) == 0  # the counters are back at zero
+        # a run that only reads another run's cache writes nothing
+        kv3 = kv2.clone()
+        got3 = ops.attention_from_qkv(qkv, hq, hk, dh, pos, seg, prep, kv3, False, slots, bt, retention,
+                                      dh ** -0.5, meta(retention))
+        assert torch.equal(kv3, kv2)
+        _assert_close_to_scale(got3, want, dt)
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_decode_attention_finds_a_far_key_in_every_key_range_and_at_the_chunk_edge(ops, dt):
+    """Eight requests around 8,200 tokens: so many key ranges that the work list is longer than the GPU takes at
+    once.  One key's score stands out; the output is its value exactly where the rule lets the query see it."""
+    hq, hk, dh, ps = 40, 8, 128, 16
+    contexts = [8190 + i for i in range(8)]  # positions 8190 .. 8197
+    qkv, kv, bt, pos, seg, slots, meta = _decode_case(hq, hk, dh, ps, dt, contexts, seed=2)
+    qkv.zero_()
+    qkv[:, : hq * dh].view(len(contexts), hq, dh)[:, :, 0] = 8.0  # every query looks along element 0
+    prep = _prep(None, None, None)
+    kv[:, 0] *= 0.05
+    kv[:, 0, :, :, 0] = 0.0
+
+    def run(hot, retention):
+        k = kv.clone()
+        for i in range(len(contexts)):
+            page, off = int(bt[i, hot // ps]), hot % ps
+            k[page, 0, :, off, 0] = 8.0
+            k[page, 1].view(hk, dh, ps)[:, :, off] = 3.0
+        out = ops.attention_from_qkv(qkv, hq, hk, dh, pos, seg, prep, k, False, slots, bt, retention, 1.0,
+                                     meta(retention))
+        return [bool(v > 2.9) for v in out.float().abs().amin(dim=-1).tolist()]
+
+    for hot in (0, 127, 128, 511, 512, 4100, 8063, 8189):  # first and last range, range edges
+        assert run(hot, ("all",)) == [True] * 8, hot
+    assert run(8191, ("all",)) == [c >= 8191 for c in contexts]  # causal
+    assert run(8191, ("chunk", 8192)) == [c == 8191 for c in contexts]  # the last key of the first chunk
+    assert run(8192, ("chunk", 8192)) == [c >= 8192 for c in contexts]  # the first key of the second
+    assert run(8000, ("chunk", 8192)) == [c < 8192 for c in contexts]
+    assert run(8190 - 299, ("window", 300)) == [c == 8190 for c in contexts]
+
+
 def test_attention_refuses_a_head_size_it_cannot_do(ops):
     from jax_llm_examples_amd.ops.hip import KernelError
     q, kv, bt, pos, seg = _attention_case(2, 1, 20, 16, torch.float32, [(0, 4)])
