@@ -84,9 +84,11 @@ def llama3_frequency_correction(freq, factor, low_freq_factor, high_freq_factor,
 
 
 def rope_frequencies(head_dim, theta, scaling, dtype=torch.float32):
-    """``model.py:706-709``: ``fraction = arange(0, dh, 2) / dh``; ``1 / theta**fraction``; then the correction."""
-    fraction = torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim
-    freq = 1.0 / (torch.tensor(float(theta), dtype=torch.float32) ** fraction)
+    """``model.py:706-709``: ``fraction = arange(0, dh, 2) / dh``; ``1 / theta**fraction``; then the correction.
+    Always formed on the CPU in float32, wherever the model runs: another device's power function may round
+    the last bit differently, and a last bit of a frequency is a thousandth of a radian at position 16,000."""
+    fraction = torch.arange(0, head_dim, 2, dtype=torch.float32, device="cpu") / head_dim
+    freq = 1.0 / (torch.tensor(float(theta), dtype=torch.float32, device="cpu") ** fraction)
     if scaling:
         freq = llama3_frequency_correction(
             freq, scaling["factor"], scaling["low_freq_factor"], scaling["high_freq_factor"],
@@ -94,9 +96,18 @@ def rope_frequencies(head_dim, theta, scaling, dtype=torch.float32):
     return freq.to(dtype)
 
 
+ANGLES_IN_FLOAT32 = False
+
+
 def rope_sin_cos(positions, freq):
-    """``model.py:712-719``: ``angle[t, j] = pos[t] * freq[j]`` in float32, then sin and cos."""
-    ang = positions.to(freq.dtype)[:, None] * freq[None, :]
+    """``model.py:712-719``: ``angle[t, j] = pos[t] * freq[j]`` in float32, then sin and cos.  When the model
+    runs in float64 as the yardstick of a float32 engine, ``ANGLES_IN_FLOAT32`` keeps this one product rounded
+    to float32 as the reference computes it (at position 8,000 that rounding is 2e-4 of a radian: it belongs
+    to what is computed, not to an implementation's error); sine and cosine in the model's dtype."""
+    if ANGLES_IN_FLOAT32:
+        ang = (positions.to(torch.float32)[:, None] * freq.to(torch.float32)[None, :]).to(freq.dtype)
+    else:
+        ang = positions.to(freq.dtype)[:, None] * freq[None, :]
     return torch.sin(ang), torch.cos(ang)
 
 
@@ -123,6 +134,10 @@ def temperature_scale(positions, floor_scale, attn_scale, dtype=torch.float32):
     return 1.0 + attn_scale * torch.log1p(torch.floor((positions.to(dtype) + 1.0) / floor_scale))
 
 
+SCORE_ELEMENTS_AT_ONCE = 1 << 30  # beyond this attention() goes head by head
+TOKENS_ONE_BY_ONE = 1024  # beyond this moe_block() takes the tokens of an expert together
+
+
 def attention(q, k, v, mask, scale):
     """``model.py:774-794``: query head ``h`` uses kv head ``h // G``; scores times ``scale``;
     masked with -1e30; softmax over keys; times values.  ``q``: ``[T, Hq, dh]``, ``k, v``: ``[S, Hkv, dh]``."""
@@ -130,6 +145,15 @@ def attention(q, k, v, mask, scale):
     hk = k.shape[1]
     g = hq // hk
     q_ = q.reshape(T, hk, g, dh)
+    if hq * T * k.shape[0] > SCORE_ELEMENTS_AT_ONCE:
+        # the same, one kv head after the other (heads do not meet): the scores of all heads of a long
+        # sequence would not fit into memory together
+        out = torch.empty(T, hk, g, dh, dtype=q.dtype, device=q.device)
+        for h in range(hk):
+            qk = torch.einsum("tgd,sd->gts", q_[:, h], k[:, h]) * scale
+            qk = torch.where(mask[None], qk, torch.full_like(qk, -1e30))
+            out[:, h] = torch.einsum("gts,sd->tgd", torch.softmax(qk, dim=-1), v[:, h])
+        return out.reshape(T, hq * dh)
     qk = torch.einsum("thgd,shd->hgts", q_, k) * scale
     qk = torch.where(mask[None, None], qk, torch.full_like(qk, -1e30))
     attn = torch.softmax(qk, dim=-1)
@@ -149,8 +173,8 @@ def attention_block(x, w, prefix, cfg, layer_idx, positions):
     uses_rope = bool(cfg["no_rope_layers"][layer_idx])
     chunk = None
     if uses_rope:
-        freq = rope_frequencies(dh, cfg["rope_theta"], cfg["rope_scaling"], x.dtype)
-        sin, cos = rope_sin_cos(positions, freq)
+        freq = rope_frequencies(dh, cfg["rope_theta"], cfg["rope_scaling"], x.dtype).to(x.device)
+        sin, cos = rope_sin_cos(positions.to(x.device), freq)
         q, k = apply_rope(q, sin, cos), apply_rope(k, sin, cos)
         if cfg["use_qk_norm"]:
             q, k = rms_norm(q, None, cfg["rms_norm_eps"]), rms_norm(k, None, cfg["rms_norm_eps"])
@@ -189,12 +213,22 @@ def moe_block(x, w, prefix, cfg, forced=None):
         gates = torch.sigmoid(torch.gather(scores, 1, idx))
     gate_up, down = w[prefix + "experts.gate_up_proj"], w[prefix + "experts.down_proj"]
     out = torch.zeros_like(x)
-    for t in range(x.shape[0]):
+    if x.shape[0] > TOKENS_ONE_BY_ONE:
+        # the same sums with the tokens of an expert taken together (the reference's own oracle for its grouped
+        # product is such a loop over experts, decode_ragged_dot.py:227-236): a long sequence token by token
+        # would read every expert matrix thousands of times
         for j in range(idx.shape[1]):
-            e = int(idx[t, j])
-            xe = x[t] * gates[t, j]
-            gu = xe @ gate_up[e]
-            out[t] += (torch.nn.functional.silu(gu[:F]) * gu[F:]) @ down[e]
+            for e in torch.unique(idx[:, j]).tolist():
+                rows = (idx[:, j] == e).nonzero().squeeze(-1)
+                gu = (x[rows] * gates[rows, j:j + 1]) @ gate_up[e]
+                out[rows] += (torch.nn.functional.silu(gu[:, :F]) * gu[:, F:]) @ down[e]
+    else:
+        for t in range(x.shape[0]):
+            for j in range(idx.shape[1]):
+                e = int(idx[t, j])
+                xe = x[t] * gates[t, j]
+                gu = xe @ gate_up[e]
+                out[t] += (torch.nn.functional.silu(gu[:F]) * gu[F:]) @ down[e]
     shared = mlp_block(x, w[prefix + "shared_expert.gate_proj.weight"], w[prefix + "shared_expert.up_proj.weight"],
                        w[prefix + "shared_expert.down_proj.weight"])
     return out + shared, idx, scores

@@ -28,7 +28,8 @@ def _vocab(name):
     return c.get("text_config", c)["vocab_size"]
 
 
-def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu", record=True):
+def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu", record=True,
+           plain_dtype=torch.float32):
     """``record``: watch every step for the experts it chose (a watched step is never the replay of a recorded
     graph); without it, steps of single tokens go through the recorded decode graphs."""
     lengths = LENGTHS[name] + (LENGTHS[name][::-1] + LENGTHS[name] if mode == "mixed" else [])
@@ -45,7 +46,7 @@ def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu",
         assert all(g.pool.handed_out > g.pool.num_pages for g in runner.cache.groups)
     runner.cache.check()
     assert runner.cache.num_live() == 0 and all(g.pool.num_held == 0 for g in runner.cache.groups)
-    plain = PlainModel(folder)
+    plain = PlainModel(folder, plain_dtype)
     if plain_device != "cpu":  # (plain PyTorch all the same; the wide configuration would take minutes on the CPU)
         plain.w = {k: v.to(plain_device) for k, v in plain.w.items()}
     worst = 0.0
@@ -57,12 +58,12 @@ def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu",
             torch.set_default_device(plain_device)
             try:
                 forced = {li: ids.to(plain_device) for li, ids in forced.items()} if forced else forced
-                ref = plain.logits(toks, forced=forced, info=info).cpu()
+                ref = plain.logits(toks, forced=forced, info=info).float().cpu()
                 info = {li: (idx.cpu(), sc.cpu()) for li, (idx, sc) in info.items()}
             finally:
                 torch.set_default_device(prev)
         else:
-            ref = plain.logits(toks, forced=forced, info=info)
+            ref = plain.logits(toks, forced=forced, info=info).float()
         assert got[rid].shape == ref.shape
         assert torch.isfinite(got[rid]).all(), f"{rid}: non-finite logits (a page that was given back?)"
         err = (got[rid] - ref).abs().max(dim=-1).values / ref.abs().max()
@@ -169,8 +170,12 @@ def test_gpu_bfloat16_serving_widths(wide_model_dir, mode):
 
 @pytest.mark.gpu
 def test_gpu_float32_serving_widths(tmp_path):
+    """The plain model runs in float64 here: run in float32 on the GPU it would go through the same library
+    products as the engine's dense projections, and a reduced-precision mode of the library at inner sizes of
+    5120 to 16384 would pass unseen."""
     folder = write_tiny("W", str(tmp_path / "W32"), torch.float32)
-    _check("W", folder, "float32", "cuda:0", "mixed", reference_ops=False, plain_device="cuda:0")
+    _check("W", folder, "float32", "cuda:0", "mixed", reference_ops=False, plain_device="cuda:0",
+           plain_dtype=torch.float64)
 
 
 @pytest.mark.gpu

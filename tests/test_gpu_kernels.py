@@ -521,6 +521,27 @@ def test_float32_products_are_true_float32(ops):
         assert torch.allclose(out, torch.full_like(out, want), rtol=1e-7)
 
 
+@pytest.mark.parametrize("rows", [1, 64, 2048])
+@pytest.mark.parametrize("k", [5120, 8192, 16384])
+def test_float32_products_are_true_float32_at_serving_sizes(ops, rows, k):
+    """The shapes the dense projections really have (which algorithm a library picks depends on them), against
+    a float64 product.  Rows of 1 + 2^-12, -1, 1 + 2^-12, -1, ... times ones: every partial sum over neighbouring
+    terms is exact in float32 in whatever order it is taken, and the result is k / 2 * 2^-12; a mode that keeps
+    10 mantissa bits of the operands gives 0.  And random operands against the float64 product."""
+    nout = 384
+    a = torch.tensor([[1.0 + 2.0 ** -12, -1.0]], device=DEV).repeat(rows, k // 2)
+    b = torch.ones(nout, k, device=DEV)
+    exact = k / 2 * 2.0 ** -12
+    ar, br = _rand(rows, k, seed=11), _rand(nout, k, seed=12)
+    want = (ar.double() @ br.double().t())
+    scale = (ar.double().abs() @ br.double().abs().t())
+    for name, fn in (("linear", ops.linear), ("lm_head", ops.lm_head), ("gemm", ops.gemm)):
+        out = fn(a, b)
+        assert float((out.double() - exact).abs().max()) <= 1e-6 * exact, name
+        err = float(((fn(ar, br).double() - want).abs() / scale).max())
+        assert err < 2e-6, f"{name}: {err:.3g} of the sum of the terms' sizes"
+
+
 def test_sampling(ops, ref):
     g = torch.Generator().manual_seed(0)
     V = 1000

@@ -332,3 +332,15 @@ def test_positions_shift_only_matters_through_distances_on_rope_layers(model_dir
     assert torch.allclose(n0, n1, atol=1e-12)
     n2 = P.attention_block(x, w, "model.layers.3.", cfg, 3, torch.arange(10) + 16)
     assert not torch.allclose(n0, n2, atol=1e-6)
+
+
+def test_the_memory_lean_forms_of_attention_and_experts_are_the_same_sums(model_dirs, monkeypatch):
+    """Long sequences at serving widths go head by head and expert by expert; the results are those of the
+    forms above (which the other tests pin)."""
+    m = P.PlainModel(model_dirs["C"], torch.float64)  # two experts per token, an explicit list of expert layers
+    toks = torch.randint(0, m.cfg["vocab_size"], (90,), generator=torch.Generator().manual_seed(4)).tolist()
+    want = m.logits(toks)
+    monkeypatch.setattr(P, "SCORE_ELEMENTS_AT_ONCE", 0)
+    monkeypatch.setattr(P, "TOKENS_ONE_BY_ONE", 0)
+    got = m.logits(toks)
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-13)
