@@ -39,3 +39,11 @@ def model_dirs_bf16(tmp_path_factory):
 
     root = tmp_path_factory.mktemp("models_bf16")
     return {name: write_tiny(name, str(root / name), torch.bfloat16) for name in TINY}
+
+
+@pytest.fixture(scope="session")
+def wide_model_dir_f32(tmp_path_factory):
+    """The two-layer model at serving widths in float32 (about 6 GB: written once for all tests that use it)."""
+    from tiny_configs import write_tiny
+
+    return write_tiny("W", str(tmp_path_factory.mktemp("models_wide_f32") / "W"), torch.float32)

@@ -29,24 +29,30 @@ def _vocab(name):
 
 
 def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu", record=True,
-           plain_dtype=torch.float32):
+           plain_dtype=torch.float32, lengths=None, max_requests=8):
     """``record``: watch every step for the experts it chose (a watched step is never the replay of a recorded
     graph); without it, steps of single tokens go through the recorded decode graphs."""
-    lengths = LENGTHS[name] + (LENGTHS[name][::-1] + LENGTHS[name] if mode == "mixed" else [])
+    if lengths is None:
+        lengths = LENGTHS[name] + (LENGTHS[name][::-1] + LENGTHS[name] if mode == "mixed" else [])
     reqs = traces.random_requests(_vocab(name), lengths, seed=5)
-    steps = MODES[mode](reqs)
+    steps = MODES[mode](reqs) if isinstance(mode, str) else mode(reqs)
     runner = make_runner(folder, dtype, traces.max_live_tokens(steps), device, reference_ops=reference_ops,
-                         poison=True)
+                         poison=True, max_requests=max_requests)
     if record:
         got, routes = traces.run_trace(runner, steps, record_routing=True)
     else:
         got, routes = traces.run_trace(runner, steps), {}
         assert runner.graphs is not None and runner.graphs.replays > 0 and runner.graphs.captures > 0
-    if mode == "mixed":  # so few pages that they were used again
+    if mode == "mixed" or not isinstance(mode, str):  # so few pages that they were used again
         assert all(g.pool.handed_out > g.pool.num_pages for g in runner.cache.groups)
     runner.cache.check()
     assert runner.cache.num_live() == 0 and all(g.pool.num_held == 0 for g in runner.cache.groups)
+    import plain_llama4
     plain = PlainModel(folder, plain_dtype)
+    plain_llama4.ANGLES_IN_FLOAT32 = plain_dtype == torch.float64  # (the yardstick of a float32 run: see there)
+    one_by_one = plain_llama4.TOKENS_ONE_BY_ONE
+    if plain_device != "cpu":
+        plain_llama4.TOKENS_ONE_BY_ONE = 48  # (on the GPU a loop over tokens costs a launch per step: by expert sooner)
     if plain_device != "cpu":  # (plain PyTorch all the same; the wide configuration would take minutes on the CPU)
         plain.w = {k: v.to(plain_device) for k, v in plain.w.items()}
     worst = 0.0
@@ -73,6 +79,8 @@ def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu",
         if dtype == "float32" and rid in routes:  # float32: the same experts, always
             for li, (idx, _) in info.items():
                 assert torch.equal(routes[rid][li].long(), idx), f"{rid} layer {li}: expert choice differs"
+    plain_llama4.ANGLES_IN_FLOAT32 = False
+    plain_llama4.TOKENS_ONE_BY_ONE = one_by_one
     return worst
 
 
@@ -169,12 +177,31 @@ def test_gpu_bfloat16_serving_widths(wide_model_dir, mode):
 
 
 @pytest.mark.gpu
-def test_gpu_float32_serving_widths(tmp_path):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sixty_four_live_requests_at_serving_widths(wide_model_dir, wide_model_dir_f32, dtype):
+    """What the benchmark's batches look like: 64 requests live at once, eight of them past 2,000 tokens, so
+    that the decode steps' key ranges are more than the GPU takes in one go; steps of 64 single tokens (64 rows
+    through the weight-streaming products, the output head and the library's dense projections), portions of
+    up to 300 tokens beside them, pages used again.  In float32 the steps of single tokens are replays of
+    recorded graphs and the yardstick is the plain model in float64; in bfloat16 the plain model is given the
+    engine's expert choices (a watched step runs launch by launch, through the same kernels)."""
+    folder = wide_model_dir if dtype == "bfloat16" else wide_model_dir_f32
+    g = torch.Generator().manual_seed(12)
+    lengths = torch.randint(100, 300, (64,), generator=g).tolist()
+    for i in range(0, 64, 8):
+        lengths[i] = 2050 + 19 * i
+    mode = lambda reqs: traces.mixed(reqs, seed=3, max_live=64, decode_tail=20, max_portion=300)
+    _check("W", folder, dtype, "cuda:0", mode, reference_ops=False, plain_device="cuda:0",
+           record=dtype == "bfloat16", plain_dtype=torch.float64 if dtype == "float32" else torch.float32,
+           lengths=lengths, max_requests=64)
+
+
+@pytest.mark.gpu
+def test_gpu_float32_serving_widths(wide_model_dir_f32):
     """The plain model runs in float64 here: run in float32 on the GPU it would go through the same library
     products as the engine's dense projections, and a reduced-precision mode of the library at inner sizes of
     5120 to 16384 would pass unseen."""
-    folder = write_tiny("W", str(tmp_path / "W32"), torch.float32)
-    _check("W", folder, "float32", "cuda:0", "mixed", reference_ops=False, plain_device="cuda:0",
+    _check("W", wide_model_dir_f32, "float32", "cuda:0", "mixed", reference_ops=False, plain_device="cuda:0",
            plain_dtype=torch.float64)
 
 

@@ -111,6 +111,69 @@ def test_command_line(model_dirs, capsys):
     assert [l["tokens"] for l in lines] == [_greedy(plain, [5, 6, 7, 8], 6), _greedy(plain, [9], 6)]
 
 
+def _assert_near_greedy(plain, prompt, out, tol=4e-2):
+    """Every generated token is the plain model's first choice after the same tokens, or within bfloat16's
+    rounding of it (``tol`` of the row's largest logit): a near-tie may fall the other way, a wrong token not."""
+    logits = plain.logits(list(prompt) + list(out))
+    for i, tok in enumerate(out):
+        row = logits[len(prompt) + i - 1]
+        assert float(row.max() - row[tok]) <= tol * float(row.abs().max()), (i, tok, int(row.argmax()))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_in_bfloat16(model_dirs_bf16, name):
+    """Through the scheduler, with steps of single tokens replayed from recorded graphs; and the same tokens
+    when every step is run launch by launch."""
+    plain = PlainModel(model_dirs_bf16[name])
+    V = plain.cfg["vocab_size"]
+    g = torch.Generator().manual_seed(3)
+    prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (5, 61, 1, 33, 17, 2)]
+    outs = {}
+    for graphs in (True, False):
+        eng = _engine(model_dirs_bf16[name], "cuda:0", "bfloat16", cache_tokens=320, decode_batch_size=4,
+                      max_num_batched_tokens=48, decode_graphs=graphs)
+        outs[graphs] = eng.generate(prompts, SamplingParams(max_decode_length=12))
+        assert (eng.runner.graphs is not None and eng.runner.graphs.replays > 0) if graphs else eng.runner.graphs is None
+        eng.cache.check()
+        assert eng.cache.num_live() == 0
+    assert outs[True] == outs[False]
+    for p, o in zip(prompts, outs[True]):
+        assert len(o) == 12
+        _assert_near_greedy(plain, p, o)
+
+
+@pytest.mark.gpu
+def test_generation_ends_at_the_context_limit(model_dirs):
+    """``max_seq_len`` (by default the configuration's max_position_embeddings): reason "length", no position
+    beyond it is ever computed."""
+    eng = _engine(model_dirs["A"], "cuda:0", cache_tokens=256, decode_batch_size=2, max_num_batched_tokens=32,
+                  max_seq_len=40)
+    a = eng.add_request(list(range(1, 31)), SamplingParams(max_decode_length=64))
+    b = eng.add_request([7, 8, 9], SamplingParams(max_decode_length=5))
+    while eng.scheduler.has_work():
+        eng.step()
+    assert (len(a.prompt) + len(a.output), a.finish_reason) == (40, "length")
+    assert (len(b.output), b.finish_reason) == (5, "length")
+    with pytest.raises(ValueError, match="longer than max_seq_len"):
+        eng.add_request(list(range(41)))
+
+
+@pytest.mark.gpu
+def test_command_line_in_bfloat16_with_pools_sized_from_free_memory(model_dirs_bf16, capsys, tmp_path):
+    from jax_llm_examples_amd.main import main
+    plain = PlainModel(model_dirs_bf16["B"])
+    rc = main(["--ckpt-path", model_dirs_bf16["B"], "--dtype", "bfloat16", "--prompt-ids", "5,6,7,8", "--prompt-ids",
+               "9", "--max-decode-length", "6", "--decode-batch-size", "2", "--max-seq-len", "64",
+               "--kv-memory-fraction", "0.0005", "--profile", str(tmp_path / "prof")])
+    assert rc == 0
+    lines = [json.loads(l) for l in capsys.readouterr().out.strip().splitlines()]
+    for prompt, l in zip(([5, 6, 7, 8], [9]), lines):
+        assert len(l["tokens"]) == 6
+        _assert_near_greedy(plain, prompt, l["tokens"])
+    assert os.path.exists(tmp_path / "prof" / "generate_trace.json")
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(model_dirs_bf16, tmp_path, dtype):

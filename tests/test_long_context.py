@@ -76,15 +76,14 @@ def test_sixteen_thousand_tokens(tmp_path, dtype):
         assert err[p] <= tol
 
 
-def test_serving_widths_float32_mixed_batches_across_the_chunk_boundaries(tmp_path):
+def test_serving_widths_float32_mixed_batches_across_the_chunk_boundaries(wide_model_dir_f32):
     """The layer sizes that serving runs at, in float32, with three requests of up to 16,500 tokens: prompts
     fed in portions of 2,048 tokens while other requests decode in the same steps; positions 8191 / 8192 and
     16383 / 16384 (the chunk's edge on the rotary layer, the temperature's step on the other) are crossed
     inside a portion by some requests and by single tokens by others; the page pools are so small that pages a
     chunk has released are taken by another request; freed pages are poisoned.  Against the plain model in
     float64."""
-    from tiny_configs import write_tiny
-    folder = write_tiny("W", str(tmp_path / "W32"), torch.float32)
+    folder = wide_model_dir_f32
     V = 20008
     g = torch.Generator().manual_seed(21)
     lengths = {"a": 16500, "b": 8300, "c": 16420}

@@ -46,10 +46,10 @@ def portions(requests, sizes=PORTIONS):
     return steps
 
 
-def mixed(requests, seed=0, max_live=4, decode_tail=24):
+def mixed(requests, seed=0, max_live=4, decode_tail=24, max_portion=19):
     """Up to ``max_live`` requests at a time; each step takes from every live request either a
-    portion (2..19 tokens) or, in its last ``decode_tail`` tokens, one token; now and then a
-    request sits a step out."""
+    portion (2..``max_portion`` tokens) or, in its last ``decode_tail`` tokens, one token; now and
+    then a request sits a step out."""
     rng = random.Random(seed)
     waiting = list(requests.items())
     live = {}
@@ -64,7 +64,7 @@ def mixed(requests, seed=0, max_live=4, decode_tail=24):
             if len(live) > 1 and rng.random() < 0.15:
                 continue
             left = len(toks) - o
-            n = 1 if left <= decode_tail else min(rng.randint(2, 19), left - decode_tail)
+            n = 1 if left <= decode_tail else min(rng.randint(2, max_portion), left - decode_tail)
             entries.append({"id": rid, "tokens": toks[o:o + n], "want": list(range(n))})
             live[rid][1] = o + n
             if o + n == len(toks):
