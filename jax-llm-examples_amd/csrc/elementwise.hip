@@ -1,9 +1,9 @@
 // Embedding gather, residual add + RMS norm, SiLU*up, row gather, expert output combine.
 #include "common.h"
+#include "rows.h"
 
 using namespace jle;
 
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 // ------------------------------------------------------------------ embedding
 template <typename T>
@@ -30,25 +30,6 @@ JLE_API int jle_embed(const int* tok, const void* table, int is_bf16, float* out
 //   delta[n] = sum_j routed[inv[n * k + j]] + shared[n]
 // One block per row.  Rows up to 8192 wide stay in registers (THREADS * EPT elements); wider rows
 // are read twice.  The sum of squares is formed in a fixed order that depends on the width only.
-template <typename DT>
-struct Delta {
-  const DT* plain;    // [N, D] or null
-  const DT* routed;   // [M, D] or null
-  const int* inv;     // [N * k]
-  const DT* shared;   // [N, D] or null
-  int k;
-  __device__ __forceinline__ bool any() const { return plain != nullptr || routed != nullptr; }
-  __device__ __forceinline__ float at(size_t n, int d, int D) const {
-    float v = 0.f;
-    if (plain != nullptr) v = Num<DT>::load(plain + n * D + d);
-    if (routed != nullptr) {
-      for (int j = 0; j < k; ++j) v += Num<DT>::load(routed + (size_t)inv[n * k + j] * D + d);
-      if (shared != nullptr) v += Num<DT>::load(shared + n * D + d);
-    }
-    return v;
-  }
-};
-
 template <typename DT, typename OT, int THREADS, int EPT>
 __global__ __launch_bounds__(THREADS) void add_rmsnorm_reg_kernel(float* __restrict__ x, Delta<DT> delta,
                                                                   const float* __restrict__ w, float eps,
@@ -85,64 +66,6 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_reg_kernel(float* __restr
       if (out32 != nullptr) out32[base + d] = h;
     }
   }
-}
-
-// four neighbouring elements
-template <typename T>
-__device__ __forceinline__ f32x4_t load4(const T* p);
-template <>
-__device__ __forceinline__ f32x4_t load4<float>(const float* p) {
-  return *reinterpret_cast<const f32x4_t*>(p);
-}
-template <>
-__device__ __forceinline__ f32x4_t load4<bf16_t>(const bf16_t* p) {
-  const uint2 r = *reinterpret_cast<const uint2*>(p);
-  return f32x4_t{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
-                 __uint_as_float(r.y & 0xffff0000u)};
-}
-// the same for data that this launch reads once and the caches need not keep
-typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
-template <typename T>
-__device__ __forceinline__ f32x4_t load4_once(const T* p);
-template <>
-__device__ __forceinline__ f32x4_t load4_once<float>(const float* p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
-}
-template <>
-__device__ __forceinline__ f32x4_t load4_once<bf16_t>(const bf16_t* p) {
-  const u32x2_t r = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
-  return f32x4_t{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
-                 __uint_as_float(r.y & 0xffff0000u)};
-}
-template <typename T>
-__device__ __forceinline__ void store4(T* p, f32x4_t v);
-template <>
-__device__ __forceinline__ void store4<float>(float* p, f32x4_t v) {
-  *reinterpret_cast<f32x4_t*>(p) = v;
-}
-template <>
-__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v) {
-  *reinterpret_cast<uint2*>(p) = uint2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-}
-
-// STREAM: the step is so large that what this launch reads and writes will have left the caches before anyone
-// wants it again (loads and stores that the caches need not keep); a step of few tokens is better off finding the
-// residual in the cache half a layer later.
-template <bool STREAM, typename T>
-__device__ __forceinline__ f32x4_t load4_as(const T* p) {
-  return STREAM ? load4_once<T>(p) : load4<T>(p);
-}
-
-template <bool STREAM, typename DT>
-__device__ __forceinline__ f32x4_t delta_at4(const Delta<DT>& delta, size_t n, int d, int D) {
-  f32x4_t v = {0.f, 0.f, 0.f, 0.f};
-  if (delta.plain != nullptr) v = load4_as<STREAM, DT>(delta.plain + n * D + d);
-  if (delta.routed != nullptr) {
-    for (int j = 0; j < delta.k; ++j)
-      v += load4_as<STREAM, DT>(delta.routed + (size_t)delta.inv[n * delta.k + j] * D + d);
-    if (delta.shared != nullptr) v += load4_as<STREAM, DT>(delta.shared + n * D + d);
-  }
-  return v;
 }
 
 // Rows whose width is a multiple of 8 (and 16-byte aligned arrays): a thread takes CPT pieces of 4

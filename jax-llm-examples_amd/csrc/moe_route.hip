@@ -1,6 +1,7 @@
 // Router: float32 logits, the k largest per token (lowest index first among equals),
 // gate = sigmoid(logit); and the stable grouping of (token, choice) pairs by expert.
 #include "common.h"
+#include "rows.h"
 
 using namespace jle;
 
@@ -76,7 +77,18 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const float* __restrict
     }
 }
 
+// A float written to / read from where all compute units of the GPU see it at once (the caches of one die are
+// written through and read past): for data that blocks on different dies hand each other within a launch.
+__device__ __forceinline__ void put_shared(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float get_shared(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // The k largest logits of token n (lowest index first among equals) and their sigmoids.
+// ACROSS: the logits were written by other blocks of this same launch (see put_shared).
+template <bool ACROSS = false>
 __device__ __forceinline__ void topk_of_token(const float* __restrict__ logits, size_t n, int E, int k,
                                               int (&best_i)[kMaxTopK], float (&gate)[kMaxTopK]) {
   float best_v[kMaxTopK];
@@ -86,7 +98,7 @@ __device__ __forceinline__ void topk_of_token(const float* __restrict__ logits, 
     best_i[j] = -1;
   }
   for (int e = 0; e < E; ++e) {
-    float v = logits[n * E + e];
+    float v = ACROSS ? get_shared(logits + n * E + e) : logits[n * E + e];
     // insert into the sorted list; strict '>' keeps the lower index ahead among equals,
     // and everything behind the insertion point moves down by one
     int ci = e;
@@ -212,6 +224,134 @@ __global__ __launch_bounds__(1024) void moe_topk_align_kernel(const float* __res
   align_by_block(ids_s, gates_s, smem, smem + E, offsets, sorted_token, sorted_gate, inv, M, E, k, extra);
 }
 
+// Steps of few tokens: the addition of the pending branch output to the residual, the norm of the sum, the
+// router's logits, the choice of experts and the grouping of the choices, in one launch.  A block is (token,
+// four experts): it forms the token's normed row (every block of a token the same row, with the arithmetic of
+// add_rmsnorm_vec_kernel: the same bits), keeps it in shared memory, and each of its wavefronts adds up one
+// expert's logit (the arithmetic of moe_logits_kernel<1, 1, true>).  The block of a token's first four experts
+// also writes the new residual and the normed row.  The block that finishes last (a ticket counter, zero between
+// launches) chooses and groups for all tokens.  N <= 256, D a multiple of 8 in (1024, 8192].
+template <typename DT, typename OT>
+__global__ __launch_bounds__(256) void norm_route_kernel(const float* __restrict__ x, Delta<DT> delta,
+                                                         const float* __restrict__ w, float eps,
+                                                         float* __restrict__ x_out, OT* __restrict__ h_out,
+                                                         const float* __restrict__ router,
+                                                         float* __restrict__ logits, int* __restrict__ ids,
+                                                         float* __restrict__ gates, int* __restrict__ offsets,
+                                                         int* __restrict__ sorted_token,
+                                                         float* __restrict__ sorted_gate, int* __restrict__ inv,
+                                                         int* __restrict__ ticket, int N, int D, int E, int k,
+                                                         int extra) {
+  constexpr int THREADS = 256, CPT = 8;
+  extern __shared__ int smem[];  // the normed row [D] (floats); afterwards the grouping's counters and pairs
+  float* row = reinterpret_cast<float*>(smem);
+  __shared__ float red[THREADS / 64];
+  __shared__ int last_flag;
+  const size_t n = blockIdx.x;
+  const size_t base = n * D;
+  const bool writer = blockIdx.y == 0;
+  f32x4_t wv[CPT];
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int d = (threadIdx.x + THREADS * i) * 4;
+    wv[i] = (w != nullptr && d < D) ? load4<float>(w + d) : f32x4_t{1.f, 1.f, 1.f, 1.f};
+  }
+  f32x4_t v[CPT];
+  float ss = 0.f;
+  const bool add = delta.any();
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int d = (threadIdx.x + THREADS * i) * 4;
+    v[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (d < D) {
+      v[i] = load4<float>(x + base + d);
+      if (add) v[i] += delta_at4<false, DT>(delta, n, d, D);
+      if (writer) store4<float>(x_out + base + d, v[i]);
+      ss += v[i][0] * v[i][0];
+      ss += v[i][1] * v[i][1];
+      ss += v[i][2] * v[i][2];
+      ss += v[i][3] * v[i][3];
+    }
+  }
+  const float tot = block_sum<THREADS>(ss, red);
+  const float rs = 1.0f / sqrtf(tot / (float)D + eps);
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int d = (threadIdx.x + THREADS * i) * 4;
+    if (d < D) {
+      f32x4_t h = v[i] * rs;
+      if (w != nullptr) h *= wv[i];
+      *reinterpret_cast<f32x4_t*>(row + d) = h;
+      if (writer && h_out != nullptr) store4<OT>(h_out + base + d, h);
+    }
+  }
+  __syncthreads();
+  // one expert's logit per wavefront
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.y * 4 + wave_index();
+  if (e < E) {
+    const float* we = router + (size_t)e * D;
+    const int D4 = D >> 2;
+    constexpr int U = 8;
+    float acc = 0.f;
+    for (int c0 = lane; c0 < D4; c0 += 64 * U) {
+      float4 rv[U], xv[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int c = min(c0 + 64 * u, D4 - 1);
+        rv[u] = *reinterpret_cast<const float4*>(we + 4 * c);
+        xv[u] = *reinterpret_cast<const float4*>(row + 4 * c);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (c0 + 64 * u < D4) {
+          acc += xv[u].x * rv[u].x;
+          acc += xv[u].y * rv[u].y;
+          acc += xv[u].z * rv[u].z;
+          acc += xv[u].w * rv[u].w;
+        }
+      }
+    }
+    const float val = wave_sum(acc);
+    if (lane == 0) put_shared(logits + n * E + e, val);
+  }
+  // the last block to get here chooses and groups: the logits were written through to where every compute unit
+  // reads them; once a block's writes are done (the fence waits for them, the barrier for all its wavefronts)
+  // it takes a ticket
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int total = (int)(gridDim.x * gridDim.y);
+    const int t = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last_flag = t == total - 1;
+    if (last_flag) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!last_flag) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  int* ismem = smem;  // counts[E], starts[E + 1], ids[N * k], gates[N * k]
+  const int M = N * k;
+  int* ids_s = ismem + 2 * E + 1;
+  float* gates_s = reinterpret_cast<float*>(ids_s + M);
+  const int t = threadIdx.x;
+  if (t < N) {
+    int best_i[kMaxTopK];
+    float gate[kMaxTopK];
+    topk_of_token<true>(logits, (size_t)t, E, k, best_i, gate);
+#pragma unroll
+    for (int j = 0; j < kMaxTopK; ++j) {
+      if (j < k) {
+        ids[t * k + j] = best_i[j];
+        gates[t * k + j] = gate[j];
+        ids_s[t * k + j] = best_i[j];
+        gates_s[t * k + j] = gate[j];
+      }
+    }
+  }
+  __syncthreads();
+  align_by_block(ids_s, gates_s, ismem, ismem + E, offsets, sorted_token, sorted_gate, inv, M, E, k, extra);
+}
+
 static int launch_logits(const float* h, const float* w, float* logits, int N, int D, int E, hipStream_t s) {
   const bool vec = D % 4 == 0 && (((uintptr_t)h | (uintptr_t)w) & 15) == 0;
   // few rows: a wavefront per (token, expert) keeps more of them in flight; many: a wavefront takes 2 tokens
@@ -275,4 +415,41 @@ JLE_API int jle_moe_align(const int* ids, const float* gates, int* offsets, int*
   if (M <= 0) return 0;
   if (E < 1 || E > 4096 || k < 1 || M % k) return JLE_BAD_ARG;
   return launch_align(ids, gates, offsets, sorted_token, sorted_gate, inv, M, E, k, extra_group ? M / k : 0, s);
+}
+
+// add + norm + router + choice + grouping in one launch, for steps of at most 256 tokens (see norm_route_kernel).
+// delta_kind: 0 none, 1 plain (delta), 2 expert sum (routed, inv_in, k_in, shared), as for jle_add_rmsnorm.
+// x_out: the residual after the addition (another array than x: the blocks of a token read x while one writes).
+// ticket: one counter, zero before the first launch and after every launch.
+// Returns JLE_BAD_ARG for sizes the fused kernel does not take (the caller then uses the separate kernels).
+JLE_API int jle_norm_route(const float* x, int delta_kind, const void* delta, const void* routed, const int* inv_in,
+                           int k_in, const void* shared, int delta_is_bf16, const float* w, float eps, float* x_out,
+                           void* h_out, int out_is_bf16, const float* router, float* logits, int* ids, float* gates,
+                           int* offsets, int* sorted_token, float* sorted_gate, int* inv, int* ticket, int N, int D,
+                           int E, int k, int extra_group, hipStream_t s) {
+  if (N <= 0) return 0;
+  if (N > 256 || D % 8 || D <= 1024 || D > 8192 || k < 1 || k > kMaxTopK || k > E || E > 4096) return JLE_BAD_ARG;
+  const uintptr_t all = (uintptr_t)x | (uintptr_t)delta | (uintptr_t)routed | (uintptr_t)shared | (uintptr_t)w |
+                        (uintptr_t)x_out | (uintptr_t)h_out | (uintptr_t)router;
+  if ((all & 15) != 0 || ticket == nullptr || logits == nullptr || x_out == x) return JLE_BAD_ARG;
+  const size_t words = (size_t)2 * E + 1 + (size_t)2 * N * k;
+  const size_t lds = (words > (size_t)D ? words : (size_t)D) * sizeof(float);
+  if (lds > 48 * 1024) return JLE_BAD_ARG;
+  dim3 g(N, (E + 3) / 4), b(256);
+#define GO(DT, OT)                                                                                               \
+  do {                                                                                                           \
+    Delta<DT> dl = {delta_kind == 1 ? (const DT*)delta : nullptr,                                                \
+                    delta_kind == 2 ? (const DT*)routed : nullptr, inv_in, (const DT*)shared, k_in};             \
+    hipLaunchKernelGGL((norm_route_kernel<DT, OT>), g, b, lds, s, x, dl, w, eps, x_out, (OT*)h_out, router,      \
+                       logits, ids, gates, offsets, sorted_token, sorted_gate, inv, ticket, N, D, E, k,          \
+                       extra_group ? N : 0);                                                                     \
+  } while (0)
+  if (delta_is_bf16) {
+    if (out_is_bf16) GO(bf16_t, bf16_t); else GO(bf16_t, float);
+  } else {
+    if (out_is_bf16) GO(float, bf16_t); else GO(float, float);
+  }
+#undef GO
+  JLE_LAUNCH_CHECK();
+  return 0;
 }

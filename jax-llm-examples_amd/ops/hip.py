@@ -29,6 +29,8 @@ _SIGNATURES = {
     "jle_paged_attention_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
                                     _vp, _vp],
     "jle_moe_route": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "jle_norm_route": [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _f, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                       _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_moe_route_align": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
@@ -57,6 +59,34 @@ class ExpertSum:
         self.routed, self.inv, self.k, self.shared = routed, inv, k, shared
         self.shape = torch.Size((n, d))
         self.dtype = routed.dtype
+
+
+class PendingNorm:
+    """The rows a norm will give, not computed yet: the residual, the branch output still to be added to it, the
+    norm's weight and eps.  Whoever consumes it computes it - inside its own launch where a kernel can (the
+    router of a step of few tokens does), else with the norm's own kernel (:meth:`rows`).  ``x_out`` is the
+    residual after the addition, ``h`` / ``h32`` the normed rows in the run dtype / float32, once computed."""
+
+    def __init__(self, ops, x, delta, weight, eps: float, out_dtype) -> None:
+        self.ops, self.x, self.delta, self.weight, self.eps = ops, x, delta, weight, float(eps)
+        self.dtype, self.shape, self.device = out_dtype, x.shape, x.device
+        self.x_out = self.h = self.h32 = None
+
+    @property
+    def done(self) -> bool:
+        return self.x_out is not None
+
+    def rows(self, want32: bool = False):
+        if not self.done:
+            self.h, self.h32 = self.ops.add_rmsnorm(self.x, self.delta, self.weight, self.eps, self.dtype, want32=True)
+            self.x_out = self.x  # (added in place)
+        if want32 and self.h32 is None:  # (computed by a kernel that kept the float32 rows to itself)
+            self.h32 = self.h.float() if self.dtype != torch.float32 else self.h
+        return self.h32 if want32 else self.h
+
+    def residual(self):
+        self.rows()
+        return self.x_out
 
 
 _LIB = None
@@ -166,6 +196,15 @@ class HipOps:
                    float(eps), _p(out), self._is_bf16(out), _p(out32), n, d)
         return out, out32
 
+    def defer_norm(self, x, delta, weight, eps: float, out_dtype) -> PendingNorm:
+        """``add_rmsnorm`` put off until a consumer asks for the rows (see :class:`PendingNorm`).  Only for
+        consumers that say they take one."""
+        return PendingNorm(self, x, delta, weight, eps, out_dtype)
+
+    @staticmethod
+    def _rows(h, want32: bool = False):
+        return h.rows(want32) if isinstance(h, PendingNorm) else h
+
     def materialize(self, delta):
         """The tensor an :class:`ExpertSum` stands for (float32)."""
         if not isinstance(delta, ExpertSum):
@@ -195,6 +234,7 @@ class HipOps:
     def linear(self, h, w, out_dtype=None):
         """``h @ w.T``: through the BLAS library (float32: true float32); a few bfloat16 rows through the
         weight-streaming kernel, which is as fast there or faster and much cheaper to launch."""
+        h = self._rows(h)
         if (h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_LINEAR_ROWS and w.dim() == 2
                 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and h.is_contiguous() and w.is_contiguous()):
             out = self.gemm_skinny(h, w)
@@ -204,6 +244,7 @@ class HipOps:
 
     def swiglu_linear(self, h, w_gate_up):
         """``silu(h @ Wg.T) * (h @ Wu.T)`` with ``w_gate_up`` = gate rows, then up rows."""
+        h = self._rows(h)
         if h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_DENSE_ROWS and h.shape[1] % 8 == 0:
             return self.gemm_skinny(h, w_gate_up, swiglu=True)
         return self.silu_mul(torch.matmul(h, w_gate_up.t()))
@@ -370,7 +411,7 @@ class HipOps:
         ps = kv_cache.shape[3]
         group = hq // max(hk, 1)
         if (meta is not None and meta.decode_bucket is not None and qkv.dtype == torch.bfloat16 and prep.plain
-                and group <= 32 and n * hk <= self.TICKETS and 4 * (dh + 4 * group * (dh + 2)) <= 48 * 1024
+                and group <= 32 and n * hk < self.TICKETS and 4 * (dh + 4 * group * (dh + 2)) <= 48 * 1024
                 and self.lib.jle_attention_mfma_supported(dh, hq, hk, ps)):
             self._chk(qkv, kv_cache.dtype, (n, (hq + 2 * hk) * dh), "q|k|v")
             self._chk(kv_cache, None, (kv_cache.shape[0], 2, hk, ps, dh), "kv pages")
@@ -564,6 +605,12 @@ class HipOps:
         the same call; ``moe_experts`` takes it as ``grouping``."""
         n, d = h32.shape
         e = router.shape[0]
+        if isinstance(h32, PendingNorm):
+            fused = None if h32.done or not group else self._norm_route(h32, router, top_k)
+            if fused is not None:
+                ids, gates, logits, grouping = fused
+                return (ids, gates, logits, grouping) if want_logits else (ids, gates, grouping)
+            h32 = h32.rows(want32=True)
         self._chk(h32, torch.float32, None, "router input")
         self._chk(router, torch.float32, (e, d), "router matrix")
         if not 1 <= top_k <= min(8, e) or e > 4096:
@@ -586,6 +633,49 @@ class HipOps:
         self._call("jle_moe_route", _p(h32), _p(router), _p(ids), _p(gates), _p(logits), n, d, e, top_k)
         return (ids, gates, logits) if want_logits else (ids, gates)
 
+    NORM_ROUTE_ROWS = 256
+
+    def _norm_route(self, pending: PendingNorm, router, top_k: int):
+        """The pending addition and norm, the router's logits, the choice and the grouping (with the extra group
+        of a shared expert's rows) in one launch, for a step of few tokens; ``None`` if the sizes do not fit."""
+        x, delta = pending.x, pending.delta
+        n, d = x.shape
+        e = router.shape[0]
+        words = 2 * e + 1 + 2 * n * top_k
+        if (n > self.NORM_ROUTE_ROWS or d % 8 or not 1024 < d <= 8192 or not 1 <= top_k <= min(8, e) or e > 4096
+                or 4 * max(words, d) > 48 * 1024 or x.dtype != torch.float32 or router.dtype != torch.float32):
+            return None
+        kind, plain, routed, inv_in, k_in, shared, is_bf16 = 0, None, None, None, 0, None, 0
+        if isinstance(delta, ExpertSum):
+            kind, routed, inv_in, k_in, shared = 2, delta.routed, delta.inv, delta.k, delta.shared
+            is_bf16 = self._is_bf16(routed)
+        elif delta is not None:
+            self._chk(delta, None, (n, d), "branch output")
+            kind, plain, is_bf16 = 1, delta, self._is_bf16(delta)
+        tensors = [t for t in (x, plain, routed, shared, pending.weight, router) if t is not None]
+        if any(t.data_ptr() % 16 or not t.is_contiguous() for t in tensors):
+            return None
+        self._chk(router, torch.float32, (e, d), "router matrix")
+        if pending.weight is not None:
+            self._chk(pending.weight, torch.float32, (d,), "norm weight")
+        dev = x.device
+        x_out = torch.empty_like(x)
+        h = torch.empty(n, d, dtype=pending.dtype, device=dev)
+        m = n * top_k
+        ids = torch.empty(n, top_k, dtype=torch.int32, device=dev)
+        gates = torch.empty(n, top_k, dtype=torch.float32, device=dev)
+        logits = torch.empty(n, e, dtype=torch.float32, device=dev)
+        offsets = torch.empty(e + 2, dtype=torch.int32, device=dev)
+        sorted_token = torch.empty(m + n, dtype=torch.int32, device=dev)
+        sorted_gate = torch.empty(m + n, dtype=torch.float32, device=dev)
+        inv = torch.empty(m, dtype=torch.int32, device=dev)
+        self._call("jle_norm_route", _p(x), kind, _p(plain), _p(routed), _p(inv_in), k_in, _p(shared), is_bf16,
+                   _p(pending.weight), pending.eps, _p(x_out), _p(h), self._is_bf16(h), _p(router), _p(logits),
+                   _p(ids), _p(gates), _p(offsets), _p(sorted_token), _p(sorted_gate), _p(inv),
+                   self._tickets[-1:].data_ptr(), n, d, e, top_k, 1)
+        pending.x_out, pending.h = x_out, h
+        return ids, gates, logits, (offsets, sorted_token, sorted_gate, inv)
+
     def moe_align(self, expert_ids, gates, num_experts: int, extra_group: bool = False):
         """Stable grouping of the (token, choice) pairs by expert: offsets ``[E + 1]``, the token and the gate of
         every sorted row, and where each pair went.  ``extra_group``: one more group behind the experts' that
@@ -607,6 +697,7 @@ class HipOps:
     def moe_experts(self, h, expert_ids, gates, w_gate_up, w_down, shared=None, tiled: bool = False, grouping=None,
                     shared_weights=None):
         """``shared``: a shared expert's output, or ``shared_weights``: its (gate|up, down) matrices, row-major."""
+        h = self._rows(h)
         n, d = h.shape
         e, f2, _ = w_gate_up.shape
         k = expert_ids.shape[1]

@@ -142,6 +142,10 @@ class FeedForward(Part):
     logits), else ``None``.  Returns ``[N, hidden]``."""
 
     wants_float32_input = False
+    # A feed-forward that only hands ``h`` / ``h32`` on to the kernel set's products and router may say so: it
+    # is then given rows that are not computed yet (the kernel set's ``defer_norm``), which a kernel of its own
+    # may compute inside its launch.  One that touches the rows itself leaves this off.
+    accepts_deferred_norm = False
 
     def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx: Any) -> torch.Tensor:  # pragma: no cover
         raise NotImplementedError

@@ -50,5 +50,9 @@ class PreNormBlock:
     def forward(self, residual, ctx, cache) -> None:
         h, _ = self.mixer_norm.forward(residual, ctx)
         residual.add(self.mixer.forward(h, ctx, cache))
-        h, h32 = self.feed_forward_norm.forward(residual, ctx, want32=self.feed_forward.wants_float32_input)
-        residual.add(self.feed_forward.forward(h, h32, ctx))
+        ff = self.feed_forward
+        if getattr(ff, "accepts_deferred_norm", False):  # (it hands the rows to the kernel set only: see there)
+            h, h32 = self.feed_forward_norm.forward(residual, ctx, want32=ff.wants_float32_input, defer=True)
+        else:
+            h, h32 = self.feed_forward_norm.forward(residual, ctx, want32=ff.wants_float32_input)
+        residual.add(ff.forward(h, h32, ctx))

@@ -39,6 +39,9 @@ class DenseSwiGLU(FeedForward):
 @register_feed_forward("moe_sigmoid_shared")
 class MoESigmoidShared(FeedForward):
     wants_float32_input = True
+    # h and h32 go to the kernel set's router and expert products only, which take rows that are not computed yet
+    # (the router of a step of few tokens does addition, norm, logits, choice and grouping in one launch)
+    accepts_deferred_norm = True
 
     def __init__(self, spec) -> None:
         super().__init__()

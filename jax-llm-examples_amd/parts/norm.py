@@ -20,5 +20,5 @@ class RMSNorm(Norm):
             return {}
         return {"weight": ParamSpec((int(self.size),), policy="float32", init=("ones",))}
 
-    def forward(self, residual, ctx, want32: bool = False):
-        return residual.normed(ctx, self.params.get("weight"), self.eps, want32)
+    def forward(self, residual, ctx, want32: bool = False, defer: bool = False):
+        return residual.normed(ctx, self.params.get("weight"), self.eps, want32, defer)

@@ -9,8 +9,15 @@ import torch
 class Residual:
     def __init__(self, x: torch.Tensor) -> None:
         assert x.dtype == torch.float32
-        self.x = x
+        self._x = x
+        self._deferred = None  # a norm (with its addition) that its consumer has been left to compute
         self.pending = None
+
+    @property
+    def x(self) -> torch.Tensor:
+        if self._deferred is not None:
+            self._x, self._deferred = self._deferred.residual(), None
+        return self._x
 
     def add(self, delta: torch.Tensor) -> None:
         if self.pending is not None:
@@ -19,7 +26,13 @@ class Residual:
             raise ValueError(f"branch output {tuple(delta.shape)} does not match residual {tuple(self.x.shape)}")
         self.pending = delta
 
-    def normed(self, ctx, weight, eps: float, want32: bool = False):
+    def normed(self, ctx, weight, eps: float, want32: bool = False, defer: bool = False):
+        """``defer``: the part that takes the rows has said it accepts rows that are not computed yet (the
+        kernel set's ``defer_norm``): it may then do addition and norm inside a launch of its own."""
+        if defer and hasattr(ctx.ops, "defer_norm"):
+            p = ctx.ops.defer_norm(self.x, self.pending, weight, eps, ctx.dtype)
+            self.pending, self._deferred = None, p
+            return p, (p if want32 else None)
         h, h32 = ctx.ops.add_rmsnorm(self.x, self.pending, weight, eps, ctx.dtype, want32)
         self.pending = None
         return h, h32

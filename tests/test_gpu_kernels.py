@@ -379,6 +379,49 @@ def test_moe_route(ops, ref, n, d, e, k):
     assert torch.equal(ids, rid) and torch.allclose(gates, rg, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("n,d,e,k,delta", [(1, 5120, 16, 1, "experts"), (8, 5120, 16, 1, "experts"), (64, 5120, 128, 1, "plain"),
+                                           (5, 1032, 3, 2, "plain"), (256, 2048, 37, 4, "none"), (3, 8192, 5, 5, "experts")])
+def test_norm_and_router_in_one_launch_equal_the_separate_kernels(ops, dt, n, d, e, k, delta):
+    """Addition, norm, router logits, choice and grouping fused for steps of few tokens: bit for bit what the norm
+    kernel, the logits kernel and the choose-and-group kernel give one after the other."""
+    from jax_llm_examples_amd.ops.hip import ExpertSum
+    x = _rand(n, d, seed=1)
+    w = _rand(d, seed=2) + 1.0
+    router = _rand(e, d, scale=0.05, seed=3)
+    if delta == "experts":
+        m = n * 2
+        routed = _rand(m, d, dt=dt, seed=4)
+        inv = torch.randperm(m, generator=torch.Generator().manual_seed(5))[: n * 2].to(torch.int32).to(DEV)
+        dl = lambda: ExpertSum(routed, inv, 2, _rand(n, d, dt=dt, seed=6), n, d)
+    elif delta == "plain":
+        dl = lambda: _rand(n, d, dt=dt, seed=4)
+    else:
+        dl = lambda: None
+    x1, x2 = x.clone(), x.clone()
+    h_a, h32_a = ops.add_rmsnorm(x1, dl(), w, 1e-5, dt, want32=True)
+    ids_a, gates_a, logits_a, group_a = ops.moe_route(h32_a, router, k, want_logits=True, group=True)
+    pending = ops.defer_norm(x2, dl(), w, 1e-5, dt)
+    calls = []
+    inner = ops._call
+    ops._call = lambda name, *a: (calls.append(name), inner(name, *a))[1]
+    try:
+        ids_b, gates_b, logits_b, group_b = ops.moe_route(pending, router, k, want_logits=True, group=True)
+    finally:
+        ops._call = inner
+    assert calls == ["jle_norm_route"], calls
+    assert torch.equal(x2, x)  # the residual is not changed in place: its new value is another tensor
+    assert torch.equal(pending.residual(), x1) and torch.equal(pending.rows(), h_a)
+    assert torch.equal(logits_b, logits_a) and torch.equal(ids_b, ids_a) and torch.equal(gates_b, gates_a)
+    for a, b in zip(group_a, group_b):
+        assert torch.equal(a, b)
+    assert int(ops._tickets.abs().sum()) == 0
+    # sizes the fused kernel does not take go through the separate kernels, with the same results
+    wide = ops.defer_norm(_rand(2, 520, seed=1), None, None, 1e-5, dt)
+    ids_c, _, _ = ops.moe_route(wide, _rand(4, 520, seed=2), 1, group=True)
+    assert wide.done and ids_c.shape == (2, 1)
+
+
 @pytest.mark.parametrize("n,d,e,k", [(700, 320, 16, 1), (600, 90, 6, 2), (520, 64, 37, 3)])
 def test_router_logits_of_a_token_do_not_depend_on_the_batch(ops, n, d, e, k):
     """Many rows take another kernel shape than few; the sums must come out bit for bit the same, or a token's
