@@ -267,6 +267,7 @@ class HipOps:
     SKINNY_MAX_ROWS = 64  # up to here a product is a stream of the weights: the MFMA weight-streaming kernel
     SKINNY_DENSE_ROWS = 16  # the fused gate|up projection of a dense feed-forward: beyond this the BLAS library
     SKINNY_LINEAR_ROWS = 8  # plain projections (q|k|v, o, down)
+    SHARED_RIDES_ROWS = 16  # a shared expert's two products ride in the routed experts' launches as one more group
 
     def gemm_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
                     variant=0, tiled=False, b_last=None, tiled_last=False):
@@ -705,7 +706,7 @@ class HipOps:
         mfma = h.dtype == torch.bfloat16 and d % 8 == 0 and (f2 // 2) % 8 == 0
         # a step of few tokens streams the shared expert's matrices in the launches of the routed experts', as one
         # more group: the cost of such a step is the kernels' getting started, not their work
-        fuse = (shared is None and shared_weights is not None and mfma and n <= self.SKINNY_DENSE_ROWS
+        fuse = (shared is None and shared_weights is not None and mfma and n <= self.SHARED_RIDES_ROWS
                 and m <= 2 * self.SKINNY_MAX_ROWS and tuple(shared_weights[0].shape) == (f2, d)
                 and tuple(shared_weights[1].shape) == (d, f2 // 2))
         if grouping is None or (fuse and grouping[0].numel() != e + 2):
