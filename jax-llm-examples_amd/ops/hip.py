@@ -43,7 +43,6 @@ _SIGNATURES = {
                                    _i, _i, _vp, _f, _f, _f, _vp, _i, _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp],
-    "jle_gemm_rows": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -108,9 +107,6 @@ def load_library():
             fn.restype = ctypes.c_int
         lib.jle_attention_mfma_supported.argtypes = [_i, _i, _i, _i]  # a query, not a launch: no stream
         lib.jle_gemm_stream_supported.argtypes = [_i, _i, _i]
-        lib.jle_gemm_rows_workspace.argtypes = [_i, _i, _i, _i]
-        lib.jle_gemm_rows_workspace.restype = ctypes.c_longlong
-        lib.jle_gemm_rows_tickets.argtypes = [_i, _i]
         lib.jle_attention_group_waves.argtypes = []
         lib._jle_path = path
         _LIB = lib
@@ -137,7 +133,6 @@ class HipOps:
         # counters of the kernels in which the last wavefront (or block) to finish does the closing work: zero
         # between launches (whoever closes puts its counter back), so they are cleared here once
         self._tickets = torch.zeros(self.TICKETS, dtype=torch.int32, device=self.device)
-        self._row_tickets = torch.zeros(self.ROW_TICKETS, dtype=torch.int32, device=self.device)
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
         torch.set_float32_matmul_precision("highest")
@@ -240,27 +235,18 @@ class HipOps:
         """``h @ w.T``: through the BLAS library (float32: true float32); a few bfloat16 rows through the
         weight-streaming kernel, which is as fast there or faster and much cheaper to launch."""
         h = self._rows(h)
-        if (h.dtype == torch.bfloat16 and w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0
-                and h.is_contiguous() and w.is_contiguous()):
-            out = None
-            if h.shape[0] <= self.SKINNY_LINEAR_ROWS:
-                out = self.gemm_skinny(h, w)
-            elif h.shape[0] <= self.ROWS_PLAIN and self._rows_fits(w.shape[0], False):
-                out = self.gemm_rows(h, w)
-            if out is not None:
-                return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
+        if (h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_LINEAR_ROWS and w.dim() == 2
+                and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and h.is_contiguous() and w.is_contiguous()):
+            out = self.gemm_skinny(h, w)
+            return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
         out = torch.matmul(h, w.t())
         return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
 
     def swiglu_linear(self, h, w_gate_up):
         """``silu(h @ Wg.T) * (h @ Wu.T)`` with ``w_gate_up`` = gate rows, then up rows."""
         h = self._rows(h)
-        if h.dtype == torch.bfloat16 and h.shape[1] % 8 == 0 and w_gate_up.dtype == torch.bfloat16:
-            if h.shape[0] <= self.SKINNY_DENSE_ROWS:
-                return self.gemm_skinny(h, w_gate_up, swiglu=True)
-            if (h.shape[0] <= self.ROWS_MAX and w_gate_up.dim() == 2 and h.is_contiguous() and w_gate_up.is_contiguous()
-                    and self._rows_fits(w_gate_up.shape[0], True)):
-                return self.gemm_rows(h, w_gate_up, swiglu=True)
+        if h.dtype == torch.bfloat16 and h.shape[0] <= self.SKINNY_DENSE_ROWS and h.shape[1] % 8 == 0:
+            return self.gemm_skinny(h, w_gate_up, swiglu=True)
         return self.silu_mul(torch.matmul(h, w_gate_up.t()))
 
     def gemm(self, a, b, *, offsets=None, a_rows=None, scale=None, out_f32=False, rows=None):
@@ -276,34 +262,6 @@ class HipOps:
         out = torch.empty(m, nout, dtype=torch.float32 if out_f32 else a.dtype, device=a.device)
         self._call("jle_gemm_generic", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), self._is_bf16(a),
                    1 if (out_f32 or a.dtype == torch.float32) else 0, m, nout, k, g)
-        return out
-
-    # dense projections of a few dozen rows: the kernel that shares the rows between 64 weight rows (measured on the
-    # serving shapes: plain products as fast as the library's at 32 rows and faster below, slower at 64; the fused
-    # gate|up product with its activation faster up to 64)
-    ROWS_MAX = 64
-    ROWS_PLAIN = 32
-    ROW_TICKETS = 8192
-
-    def _rows_fits(self, nout: int, swiglu: bool) -> bool:
-        return int(self.lib.jle_gemm_rows_tickets(nout, int(swiglu))) <= self.ROW_TICKETS
-
-    def gemm_rows(self, a, b, *, swiglu=False):
-        """bfloat16 product of up to 64 rows with a row-major weight matrix (see ``gemm_rows.hip``); with
-        ``swiglu`` the result is ``silu(gate) * up`` of the two halves of ``b``'s rows."""
-        m, k = a.shape
-        nout = b.shape[0]
-        self._chk(a, torch.bfloat16, None, "A")
-        self._chk(b, torch.bfloat16, (nout, k), "B")
-        if m > self.ROWS_MAX or k % 8 or (swiglu and nout % 2):
-            raise KernelError(f"the product for a few dozen rows takes up to {self.ROWS_MAX} rows and an inner size "
-                              f"that is a multiple of 8, got {m} x {k}")
-        if not self._rows_fits(nout, swiglu):
-            raise KernelError(f"the product for a few dozen rows has counters for {self.ROW_TICKETS * 64} weight rows")
-        out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.bfloat16, device=a.device)
-        words = int(self.lib.jle_gemm_rows_workspace(m, nout, k, int(swiglu)))
-        part = torch.empty(max(words, 1), dtype=torch.float32, device=a.device)
-        self._call("jle_gemm_rows", _p(a), _p(b), _p(out), _p(part), _p(self._row_tickets), int(swiglu), m, nout, k)
         return out
 
     SKINNY_MAX_ROWS = 64  # up to here a product is a stream of the weights: the MFMA weight-streaming kernel

@@ -555,30 +555,6 @@ def test_product_kernel_and_lm_head(ops, ref, dt):
     _assert_close_to_scale(ops.linear(h, w), ref.linear(h, w), dt)
 
 
-@pytest.mark.parametrize("swiglu", [False, True])
-@pytest.mark.parametrize("m,nout,k", [(9, 7168, 5120), (64, 5120, 5120), (33, 5120, 8192), (64, 16384, 5120),
-                                      (17, 100, 72), (48, 96, 264), (64, 2 * 1000, 520), (20, 640, 64)])
-def test_product_for_a_few_dozen_rows(ops, swiglu, m, nout, k):
-    """Row-major weights, 64 weight rows and a slice of K per block, the slices added up by the last block to
-    finish: against a float32 product of the same bfloat16 operands, twice (the counters are back at zero)."""
-    a = _rand(m, k, dt=torch.bfloat16, seed=1)
-    w = _rand(nout, k, dt=torch.bfloat16, scale=k ** -0.5, seed=2)
-    want = a.float() @ w.float().t()
-    if swiglu:
-        f = nout // 2
-        want = torch.nn.functional.silu(want[:, :f]) * want[:, f:]
-    first = ops.gemm_rows(a, w, swiglu=swiglu)
-    _assert_close_to_scale(first, want, torch.bfloat16)
-    assert int(ops._row_tickets.abs().sum()) == 0
-    assert torch.equal(ops.gemm_rows(a, w, swiglu=swiglu), first)  # the slices are added in their order: the same bits
-    # through the entry points the parts use
-    got = ops.swiglu_linear(a, w) if swiglu else ops.linear(a, w)
-    if (ops.SKINNY_DENSE_ROWS < m <= ops.ROWS_MAX) if swiglu else (ops.SKINNY_LINEAR_ROWS < m <= ops.ROWS_PLAIN):
-        assert torch.equal(got, first)
-    else:  # (fewer rows go through the kernel for a few rows, more through the library)
-        _assert_close_to_scale(got, want, torch.bfloat16)
-
-
 def test_float32_products_are_true_float32(ops):
     # a reduced-precision matrix mode (tf32/xf32: 10 mantissa bits) would lose the small term
     a = torch.tensor([[1.0, 2.0 ** -14]], device=DEV).repeat(4, 64)  # 128 columns
