@@ -107,12 +107,14 @@ class _Recording:
 
 
 class DecodeGraphs:
-    MAX_RECORDINGS = 12
+    MAX_RECORDINGS = 16
+    RECORD_AFTER = 2  # a (requests, bound) pair is recorded when it comes the second time: one that comes once is not worth it
 
     def __init__(self, model, cache, ops) -> None:
         self.model, self.cache, self.ops = model, cache, ops
         self.recordings: "collections.OrderedDict[tuple, _Recording]" = collections.OrderedDict()
         self.pool = None
+        self.seen: "collections.Counter[tuple]" = collections.Counter()
         self.replays = 0
         self.captures = 0
         self.safe = (getattr(ops, "name", "") == "hip" and model.device.type == "cuda"
@@ -123,14 +125,20 @@ class DecodeGraphs:
         return self.safe and tap is None and all(len(e.tokens) == 1 for e in entries)
 
     @torch.no_grad()
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry]):
         """The entries hold reservations for their one token.  Returns float32 logits of the wanted rows; they
-        lie in the recording's own output buffer until the next step of the same shape."""
+        lie in the recording's own output buffer until the next step of the same shape.  ``None``: this step is
+        better run launch by launch (its shape has not come often enough to be recorded)."""
         cache, model = self.cache, self.model
         longest = max(cache.requests[e.rid].num_tokens for e in entries) + 1
         key = (len(entries), decode_bucket(longest))
         rec = self.recordings.get(key)
         if rec is None:
+            self.seen[key] += 1
+            if self.seen[key] < self.RECORD_AFTER:
+                if len(self.seen) > 4096:
+                    self.seen.clear()
+                return None
             rec = _Recording(model, cache, self.ops, *key)
             self.recordings[key] = rec
             while len(self.recordings) > self.MAX_RECORDINGS:

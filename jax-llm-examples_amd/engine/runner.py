@@ -68,10 +68,11 @@ class ModelRunner:
                 cache.free(rid)
             raise
         try:
+            logits = None
             if self.graphs is not None and self.graphs.fits(entries, tap):
                 logits = self.graphs.run(entries)
                 num_tokens = len(entries)
-            else:
+            if logits is None:
                 ctx = build_context(self.ops, self.model.dtype, self.model.device, cache, entries,
                                     self.model.plan.vocab_size, tap)
                 logits = self.model.forward(ctx, cache)
