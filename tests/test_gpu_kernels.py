@@ -226,18 +226,21 @@ def _decode_case(hq, hk, dh, ps, dt, contexts, seed=0):
     return qkv, kv, bt, pos, seg, slots, meta
 
 
-@pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("hq,hk,dh,ps,contexts", [
+_DECODE_CASES = [
     (40, 8, 128, 16, [3000 + 94 * i for i in range(64)]),  # the serving shape: 64 requests between 3,000 and 9,000
     (40, 8, 128, 16, [8191, 8192, 8193, 0, 5, 16383, 16384, 4095]),
     (10, 2, 64, 32, [0, 1, 31, 32, 700, 129]), (6, 1, 32, 16, [77]), (20, 1, 96, 48, [500, 47, 48]),
-    (34, 2, 32, 16, [260, 3]), (4, 4, 256, 16, [90, 1000])])
-@pytest.mark.parametrize("retention", [("all",), ("chunk", 8192), ("chunk", 96), ("window", 200)])
+    (34, 2, 32, 16, [260, 3]), (4, 4, 256, 16, [90, 1000])]
+_DECODE_RETENTIONS = [("all",), ("chunk", 8192), ("chunk", 96), ("window", 200)]
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("hq,hk,dh,ps,contexts,retention",
+                         [(*c, r) for c in _DECODE_CASES for r in _DECODE_RETENTIONS
+                          if r != ("chunk", 8192) or max(c[4]) >= 3000])  # (the large chunk: long contexts only)
 def test_attention_of_a_step_of_single_tokens_from_the_projection_rows(ops, ref, dt, hq, hk, dh, ps, contexts, retention):
     """Rotation, q/k norm, scale, the write of the new key and value, attention over many key ranges and their
     merge: one launch in bfloat16 (two kernels and a merge in float32), against the plain ops."""
-    if retention == ("chunk", 8192) and max(contexts) < 3000:
-        pytest.skip("the large chunk is for the long contexts")
     from jax_llm_examples_amd.ops.hip import HipOps
     qkv, kv, bt, pos, seg, slots, meta = _decode_case(hq, hk, dh, ps, dt, contexts)
     inv = (1.0 / (10000.0 ** (torch.arange(0, dh, 2).float() / dh))).to(DEV)
@@ -487,10 +490,13 @@ def test_moe_experts(ops, ref, dt, n, d, f, e, k):
     assert torch.equal(ops.gather_rows(lazy, idx), got[idx.long()])
 
 
-@pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("tiled", [False, True])
-@pytest.mark.parametrize("n,d,f,e,k", [(1, 64, 32, 4, 1), (9, 96, 48, 3, 2), (16, 256, 64, 16, 1), (17, 64, 32, 4, 1),
-                                       (50, 96, 48, 5, 1)])
+_SHARED_CASES = [(1, 64, 32, 4, 1), (9, 96, 48, 3, 2), (16, 256, 64, 16, 1), (17, 64, 32, 4, 1), (50, 96, 48, 5, 1)]
+
+
+# (the streaming layout exists for bfloat16 matrices of whole 16 x 32 tiles only)
+@pytest.mark.parametrize("dt,tiled,n,d,f,e,k",
+                         [(dt, False, *c) for dt in DT for c in _SHARED_CASES] +
+                         [(torch.bfloat16, True, *c) for c in _SHARED_CASES if c[1] % 32 == 0 and c[2] % 32 == 0])
 def test_moe_experts_with_the_shared_expert_given_by_its_matrices(ops, ref, dt, tiled, n, d, f, e, k):
     """Up to 16 tokens the shared expert's products go through the routed experts' launches as one more group
     (its matrices stay row-major beside experts in either layout); beyond, through the library.  The same sum."""
@@ -504,8 +510,7 @@ def test_moe_experts_with_the_shared_expert_given_by_its_matrices(ops, ref, dt, 
     gates = torch.rand(n, k, generator=g).to(DEV)
     want = ref.moe_experts(h, ids, gates, wgu, wd, shared_weights=(sgu, sd))
     if tiled:
-        if dt != torch.bfloat16 or not (can_tile(wgu) and can_tile(wd)):
-            pytest.skip("the streaming layout is for bfloat16 matrices of whole tiles")
+        assert can_tile(wgu) and can_tile(wd)
         wgu, wd = wgu.clone(), wd.clone()
         tile_(wgu)
         tile_(wd)
