@@ -641,17 +641,120 @@ __global__ __launch_bounds__(WAVES * 64, DH <= 128 ? 2 : 1) void attention_prefi
 // The kernel above with the keys and values of a step brought into shared memory by the load unit itself
 // (global_load_lds: a wavefront's 64 lanes fetch 16 bytes each from addresses of their own, and the kilobyte
 // lands in shared memory in lane order): no registers hold data on its way, nothing is stored to shared memory by
-// the wavefronts, and the only wait is for the loads asked for two steps earlier.  What lands contiguously
+// the wavefronts, and the only wait is for the loads asked for a step earlier.  What lands contiguously
 // decides the layout, and which piece a lane fetches makes it free of bank conflicts:
 //   keys, per tile: [16 rows][16 pieces of 16 bytes], piece p of row r at place p ^ r: the 16 lanes that read
 //     the same piece of 16 different rows meet 16 different places;
 //   values, per tile: [128 elements][2 halves of 8 keys], half h of element d at place h ^ ((d >> 3) & 1): the 16
 //     lanes that read 8 bytes each of 16 consecutive elements meet 16 different pairs of banks.
-// A buffer is 16 KB (two key tiles, two value tiles); four buffers: a step's loads are asked for three steps ahead,
-// into the buffer of the step that has just been finished by every wavefront (two steps ahead: 6 % slower at 8,192
-// tokens).  Measured against the kernel above at head size 128: 5 to 11 % faster, the same bits.
+// A step is 64 keys (four key tiles and four value tiles of 4 KB: each wavefront fetches the tile pair of its own
+// number), so that the maxima, the sums, the accumulators' correction, the barrier and the page look-up come once per
+// 64 keys; two buffers of 32 KB: a step's loads are asked for when the step before it begins, into the buffer that
+// every wavefront has just left.  Measured at head size 128 against the kernel above (32 keys a step, through
+// registers): 15 % faster at 2,048 tokens, 20 % at 8,192; with 32 keys a step and the same loads it was 5 to 11 %.
 __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t byte_off, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n" ::"v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
+}
+
+// One step of 64 keys (four tiles of 16) for the columns of a wavefront: softmax_and_values for twice the keys, so
+// that the maxima, the sums and the accumulators' correction are done once per 64 keys.  The values are taken from
+// shared memory half by half (tiles 0 and 1, then 2 and 3): sv points at the step's value tiles, v_rd is the lane's
+// offset in a tile, tile_bytes the distance between tiles.  halves: 1 if tiles 2 and 3 hold nothing for this wavefront.
+template <int DH, int CT, bool MASKED>
+__device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], const bool (&act)[4], int halves,
+                                                     const unsigned char* sv, uint32_t v_rd, int tile_bytes, int kb,
+                                                     const Columns (&col)[CT], int k_lo, int k_hi, float scale_log2,
+                                                     float (&m)[CT], float (&l)[CT], f32x4 (&acc)[CT][DH / 16]) {
+  constexpr int DT = DH / 16;
+  const int g = (threadIdx.x & 63) >> 4;
+  bf16x8 pb[CT][2];
+  float corr[CT];
+  bool unchanged = true;
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = st[ct][tt][i];
+        if (MASKED) {
+          const int key = kb + 16 * tt + 4 * g + i;
+          const bool ok = act[tt] && key >= col[ct].lo && key <= col[ct].hi;
+          v = ok ? v : -INFINITY;
+          st[ct][tt][i] = v;
+        }
+        mx = fmaxf(mx, v);
+      }
+    mx = column_max(mx);
+    const float m_new = fmaxf(m[ct], mx * scale_log2);  // the scale is positive
+    const float m_use = (MASKED && m_new == -INFINITY) ? 0.f : m_new;
+    corr[ct] = __builtin_amdgcn_exp2f(m[ct] - m_use);  // m = -inf: 0 (nothing accumulated yet)
+    unchanged = unchanged && m_new == m[ct];
+    float sum = 0.f;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      float p[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        p[j] = __builtin_amdgcn_exp2f(fmaf(st[ct][2 * hf + (j >> 2)][j & 3], scale_log2, -m_use));  // masked: exp2(-inf) = 0
+        sum += p[j];
+      }
+      const uint4 pk = {pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7])};
+      pb[ct][hf] = __builtin_bit_cast(bf16x8, pk);
+    }
+    l[ct] = l[ct] * corr[ct] + sum;
+    m[ct] = m_new;
+  }
+  if (!__all(unchanged)) {
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        acc[ct][dt][0] *= corr[ct];
+        acc[ct][dt][1] *= corr[ct];
+        acc[ct][dt][2] *= corr[ct];
+        acc[ct][dt][3] *= corr[ct];
+      }
+  }
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) {
+    if (hf >= halves) break;
+    uint4 vraw[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const uint2 t0 = *reinterpret_cast<const uint2*>(sv + (2 * hf) * tile_bytes + v_rd + dt * 512);
+      const uint2 t1 = *reinterpret_cast<const uint2*>(sv + (2 * hf + 1) * tile_bytes + v_rd + dt * 512);
+      vraw[dt] = uint4{t0.x, t0.y, t1.x, t1.y};
+    }
+    if (MASKED) {
+      // values: keys outside [k_lo, k_hi] may never have been written: they are read as zero
+      uint32_t keep[2][2];
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const int key = kb + 16 * (2 * hf + t2) + 4 * g + 2 * h2;
+          const uint32_t lo_ok = (key >= k_lo && key <= k_hi) ? 0x0000ffffu : 0u;
+          const uint32_t hi_ok = (key + 1 >= k_lo && key + 1 <= k_hi) ? 0xffff0000u : 0u;
+          keep[t2][h2] = lo_ok | hi_ok;
+        }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        vraw[dt].x &= keep[0][0];
+        vraw[dt].y &= keep[0][1];
+        vraw[dt].z &= keep[1][0];
+        vraw[dt].w &= keep[1][1];
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const bf16x8 a = __builtin_bit_cast(bf16x8, vraw[dt]);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+        acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb[ct][hf], acc[ct][dt], 0, 0, 0);
+    }
+  }
 }
 
 __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
@@ -660,10 +763,11 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
     int table_width, const int* __restrict__ tiles, const int* __restrict__ groups, int ret_mode, int ret_param,
     float scale_log2, int Hq, int Hkv, int ps) {
   constexpr int DH = 128, CT = 2, KC = DH / 32, DT = DH / 16;
-  constexpr int NB = 4;
+  constexpr int NB = 2;
   constexpr int TILE = 16 * DH * 2;  // bytes of a key tile, and of a value tile
-  constexpr int BUF = 4 * TILE;
+  constexpr int BUF = 8 * TILE;      // a step: four key tiles, four value tiles
   __shared__ __attribute__((aligned(1024))) unsigned char smem[NB * BUF];
+  __shared__ int any_bad;
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
   const int lane = threadIdx.x & 63, wave = wave_index();
   const int c16 = lane & 15, g = lane >> 4;
@@ -687,6 +791,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
   const int* table = block_table + (size_t)token_segment[n0] * table_width;
   const size_t plane = (size_t)ps * DH;
   const size_t page_stride = 2 * (size_t)Hkv * plane;
+  if (threadIdx.x == 0) any_bad = 0;
 
   Columns col[CT];
   bf16x8 qb[CT][KC];
@@ -716,93 +821,76 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
   int all_lo, all_hi;
   common_range<CT>(col, all_lo, all_hi);
 
-  // What this wavefront fetches of a step: two of the eight kilobytes of the keys and two of the values', all of
-  // key tile wave / 2.  Byte offsets from the tile's first key / first value column:
-  const int my_tile = wave >> 1;
-  const int part0 = 2 * (wave & 1);
-  uint32_t k_src[2], v_src[2];
+  // What this wavefront fetches of a step: key tile `wave` and value tile `wave`, four kilobytes each.  Byte offsets
+  // from the tile's first key / first value column:
+  uint32_t k_src[4], v_src[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int row = 4 * (part0 + i) + (lane >> 4);
+  for (int i = 0; i < 4; ++i) {
+    const int row = 4 * i + (lane >> 4);
     const int piece = (lane & 15) ^ row;
     k_src[i] = (uint32_t)(row * DH + piece * 8) * 2;
-    const int d = 32 * (part0 + i) + (lane >> 1);
+    const int d = 32 * i + (lane >> 1);
     const int hh = (lane & 1) ^ ((d >> 3) & 1);
     v_src[i] = (uint32_t)(d * ps + hh * 8) * 2;
   }
-  const uint32_t my_dst = (uint32_t)(my_tile * TILE + part0 * 1024);
   // what it reads: keys of tile tt, piece c * 4 + g of row c16; values of tile tt, keys 4 g .. 4 g + 3 of element d
   uint32_t k_rd[KC];
 #pragma unroll
   for (int c = 0; c < KC; ++c) k_rd[c] = (uint32_t)(c16 * 256 + (((c * 4 + g) ^ c16) * 16));
-  const uint32_t v_rd = (uint32_t)(2 * TILE + (c16 * 2 + ((g >> 1) ^ (c16 >> 3))) * 16 + (g & 1) * 8);  // + dt * 512
+  const uint32_t v_rd = (uint32_t)((c16 * 2 + ((g >> 1) ^ (c16 >> 3))) * 16 + (g & 1) * 8);  // + dt * 512
 
   bool bad = false;
-  const int kb_first = (k_lo / 32) * 32;
-  int next_kb = kb_first;
-  int page_index = next_kb / ps, page_off = next_kb % ps;
-  int pages[2], offs[2];
+  const int kb_first = (k_lo / 64) * 64;
+  // this wavefront's tile of the next step to ask for: its first key, and where that lies in the pages
+  int my_key = kb_first + 16 * wave;
+  int page_index = my_key / ps, page_off = my_key % ps;
+  int page = 0;
+  bool need = false;
   auto look_up = [&]() {
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      const int key0 = next_kb + 16 * tt;
-      int idx = page_index, off = page_off + 16 * tt;
-      if (off >= ps) {
-        off -= ps;
-        ++idx;
-      }
-      offs[tt] = off;
-      pages[tt] = -1;
-      if (key0 <= k_hi && key0 + 15 >= k_lo) {
-        pages[tt] = table[idx];
-        if (pages[tt] < 0) bad = true;  // the block's result is NaN
-      }
-    }
+    need = my_key <= k_hi && my_key + 15 >= k_lo;
+    page = table[min(page_index, table_width - 1)];  // (asked for now, looked at when the step's loads are asked for)
   };
   look_up();
-  // every load is asked for unconditionally (a tile that is not needed reads page 0, whose contents are then masked
-  // like any key out of range), so that the count of loads on their way is the same in every wavefront
+  // every load is asked for unconditionally (a tile that is not needed reads some page, whose contents are then
+  // masked like any key out of range), so that the count of loads on their way is the same in every wavefront
   auto load_step = [&](int buf) {
-    const int page = max(my_tile ? pages[1] : pages[0], 0);
-    const int off = my_tile ? offs[1] : offs[0];
-    const bf16_t* keys = kv + (size_t)page * page_stride + (size_t)hk * plane;
-    const bf16_t* values = keys + (size_t)Hkv * plane + off;
-    keys += (size_t)off * DH;
-    const uint32_t dst = lds0 + (uint32_t)buf * BUF + my_dst;
-    load_to_lds16(keys, k_src[0], dst);
-    load_to_lds16(keys, k_src[1], dst + 1024);
-    load_to_lds16(values, v_src[0], dst + 2 * TILE);
-    load_to_lds16(values, v_src[1], dst + 2 * TILE + 1024);
-    next_kb += 32;
-    page_off += 32;  // a page holds at least 16 keys: at most two pages further
-    if (page_off >= ps) {
-      page_off -= ps;
-      ++page_index;
-    }
-    if (page_off >= ps) {
-      page_off -= ps;
-      ++page_index;
-    }
+    if (need && page < 0) bad = true;  // the block's result is NaN
+    const bf16_t* keys = kv + (size_t)max(page, 0) * page_stride + (size_t)hk * plane;
+    const bf16_t* values = keys + (size_t)Hkv * plane + page_off;
+    keys += (size_t)page_off * DH;
+    const uint32_t dst = lds0 + (uint32_t)buf * BUF + (uint32_t)wave * TILE;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_to_lds16(keys, k_src[i], dst + i * 1024);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_to_lds16(values, v_src[i], dst + 4 * TILE + i * 1024);
+    my_key += 64;
+    page_off += 64;  // a page holds at least 16 keys: at most four pages further
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (page_off >= ps) {
+        page_off -= ps;
+        ++page_index;
+      }
     look_up();
   };
 
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the queries have come; from here on only the steps' loads count
   asm volatile("" ::: "memory");
   load_step(0);
-  load_step(1);
-  load_step(2);
   int buf = 0;
-  for (int kb = kb_first; kb <= k_hi; kb += 32) {
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");  // this step's four loads have landed (the next two steps' may be on their way)
+  for (int kb = kb_first; kb <= k_hi; kb += 64) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this step's eight loads have landed
     __syncthreads();
-    load_step(buf == 0 ? NB - 1 : buf - 1);  // the third step from here, into the buffer that every wavefront has just left
-    if (head_ok && kb + 31 >= my_lo && kb <= my_hi) {
+    load_step(buf ^ 1);  // the next step, into the buffer that every wavefront has just left
+    if (head_ok && kb + 63 >= my_lo && kb <= my_hi) {
       const unsigned char* sb = smem + buf * BUF;
-      f32x4 st[CT][2];
+      const int halves = kb + 32 <= my_hi ? 2 : 1;  // (tiles 2 and 3 lie past this wavefront's last key)
+      f32x4 st[CT][4];
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
+      for (int tt = 0; tt < 4; ++tt) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (tt >= 2 * halves) continue;
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
           const uint4 kvv = *reinterpret_cast<const uint4*>(sb + tt * TILE + k_rd[c]);
@@ -812,23 +900,22 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
             st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
         }
       }
-      uint4 vraw[DT];
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const uint2 t0 = *reinterpret_cast<const uint2*>(sb + v_rd + dt * 512);
-        const uint2 t1 = *reinterpret_cast<const uint2*>(sb + v_rd + dt * 512 + TILE);
-        vraw[dt] = uint4{t0.x, t0.y, t1.x, t1.y};
-      }
-      if (kb >= all_lo && kb + 31 <= all_hi) {  // the same for the whole wavefront
-        softmax_and_values<DH, CT, false>(st, true, true, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+      if (kb >= all_lo && kb + 63 <= all_hi) {  // the same for the whole wavefront
+        const bool act[4] = {true, true, true, true};
+        softmax64_and_values<DH, CT, false>(st, act, 2, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
       } else {
-        const bool act0 = kb <= k_hi && kb + 15 >= k_lo, act1 = kb + 16 <= k_hi && kb + 31 >= k_lo;
-        softmax_and_values<DH, CT, true>(st, act0, act1, vraw, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+        bool act[4];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) act[tt] = tt < 2 * halves && kb + 16 * tt <= k_hi && kb + 16 * tt + 15 >= k_lo;
+        softmax64_and_values<DH, CT, true>(st, act, halves, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
       }
     }
-    buf = buf == NB - 1 ? 0 : buf + 1;
+    buf ^= 1;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in shared memory after the block has gone
+  if (bad) any_bad = 1;
+  __syncthreads();
+  bad = any_bad != 0;
   if (!head_ok) return;
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
@@ -1241,7 +1328,7 @@ static bool head_dim_ok(int dh) { return dh == 32 || dh == 64 || dh == 96 || dh 
 // Wavefronts, and so (tile, head) items, per block of the key-sharing prefill kernel: one per SIMD, and two
 // such blocks fit a compute unit.
 constexpr int kGroupWaves = 4;
-static_assert(kGroupWaves == 4, "attention_prefill_lds_kernel deals a step's sixteen kilobytes to four wavefronts");
+static_assert(kGroupWaves == 4, "attention_prefill_lds_kernel deals a step's four tile pairs to four wavefronts");
 JLE_API int jle_attention_group_waves() { return kGroupWaves; }
 
 JLE_API int jle_attention_mfma_supported(int dh, int Hq, int Hkv, int ps) {
