@@ -200,13 +200,28 @@ def _attention_case(hq, hk, dh, ps, dt, seg_specs, seed=0):
 @pytest.mark.parametrize("dt", DT)
 @pytest.mark.parametrize("hq,hk,dh,ps", [(4, 2, 16, 16), (5, 1, 48, 16), (6, 3, 32, 8), (8, 8, 64, 16),
                                          (10, 2, 128, 16), (2, 1, 256, 32), (3, 1, 80, 16), (6, 3, 32, 16),
-                                         (40, 8, 128, 16), (20, 1, 96, 48), (4, 4, 256, 16), (5, 5, 64, 64)])
+                                         (40, 8, 128, 16), (20, 1, 96, 48), (4, 4, 256, 16), (5, 5, 64, 64),
+                                         (10, 2, 128, 32), (9, 3, 128, 48), (10, 5, 128, 64)])
 @pytest.mark.parametrize("retention", [("all",), ("chunk", 24), ("window", 37)])
 def test_paged_attention(ops, ref, dt, hq, hk, dh, ps, retention):
     case = _attention_case(hq, hk, dh, ps, dt, [(0, 70), (130, 1), (45, 9), (63, 2), (200, 1), (600, 1), (255, 3)])
     q, kv, bt, pos, seg = case
     got = ops.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
     want = ref.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
+    _assert_close_to_scale(got, want, dt)
+
+
+@pytest.mark.parametrize("hq,hk,ps", [(10, 2, 16), (40, 8, 16), (6, 3, 32), (9, 3, 48), (4, 2, 64)])
+@pytest.mark.parametrize("retention", [("all",), ("chunk", 192), ("chunk", 100), ("window", 150)])
+def test_paged_attention_of_long_portions_at_head_size_128(ops, ref, hq, hk, ps, retention):
+    """Portions of hundreds of tokens behind hundreds of cached ones, at the head size whose kernel takes 64 keys a
+    step straight into shared memory: many steps, pages of every size crossed inside a step, rules whose first
+    key lies inside a step and inside a page."""
+    dt = torch.bfloat16
+    case = _attention_case(hq, hk, 128, ps, dt, [(0, 333), (190, 130), (517, 1), (64, 64), (1000, 35)], seed=3)
+    q, kv, bt, pos, seg = case
+    got = ops.paged_attention(q, kv, bt, pos, seg, retention, 128 ** -0.5)
+    want = ref.paged_attention(q, kv, bt, pos, seg, retention, 128 ** -0.5)
     _assert_close_to_scale(got, want, dt)
 
 
