@@ -29,7 +29,7 @@ def _vocab(name):
 
 
 def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu", record=True,
-           plain_dtype=torch.float32, lengths=None, max_requests=8):
+           plain_dtype=torch.float32, lengths=None, max_requests=8, page_size=16):
     """``record``: watch every step for the experts it chose (a watched step is never the replay of a recorded
     graph); without it, steps of single tokens go through the recorded decode graphs."""
     if lengths is None:
@@ -37,7 +37,7 @@ def _check(name, folder, dtype, device, mode, reference_ops, plain_device="cpu",
     reqs = traces.random_requests(_vocab(name), lengths, seed=5)
     steps = MODES[mode](reqs) if isinstance(mode, str) else mode(reqs)
     runner = make_runner(folder, dtype, traces.max_live_tokens(steps), device, reference_ops=reference_ops,
-                         poison=True, max_requests=max_requests)
+                         poison=True, max_requests=max_requests, page_size=page_size)
     if record:
         got, routes = traces.run_trace(runner, steps, record_routing=True)
     else:
@@ -174,6 +174,18 @@ def test_gpu_bfloat16_serving_widths(wide_model_dir, mode):
     """Two layers (one rotary, one without) at the widths the benchmark runs: the kernel variants that only these
     sizes reach (rows of 5120, 40 heads on 8, experts 8192 wide) against the plain implementation."""
     _check("W", wide_model_dir, "bfloat16", "cuda:0", mode, reference_ops=False, plain_device="cuda:0")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("page_size", [32, 64])
+@pytest.mark.parametrize("name,dtype,mode", [("W", "bfloat16", "mixed"), ("W", "bfloat16", "portions"), ("A", "bfloat16", "mixed"),
+                                             ("C", "bfloat16", "mixed"), ("B", "float32", "mixed"), ("D", "float32", "portions")])
+def test_gpu_pages_of_other_sizes(model_dirs, model_dirs_bf16, wide_model_dir, name, dtype, mode, page_size):
+    """Pages of 32 and 64 tokens: block tables half and a quarter as wide, chunks and windows that end inside a page,
+    the kernels' walks through pages that hold more than one of their tiles."""
+    folder = wide_model_dir if name == "W" else (model_dirs_bf16 if dtype == "bfloat16" else model_dirs)[name]
+    _check(name, folder, dtype, "cuda:0", mode, reference_ops=False, plain_device="cuda:0" if name == "W" else "cpu",
+           page_size=page_size)
 
 
 @pytest.mark.gpu
