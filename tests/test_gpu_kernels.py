@@ -466,6 +466,32 @@ def test_router_and_grouping_in_one_call(ops, n, d, e, k):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("n", [511, 512, 2048])
+def test_routing_beside_the_shared_expert_gives_the_same_experts_and_sums(ops, n):
+    """From 512 tokens on a routing asked for with ``beside`` runs on a second stream while the shared expert's
+    products run on the first; the experts' products wait for it.  Several rounds, with the first stream kept busy,
+    against the same calls on one stream."""
+    d, f, e = 256, 64, 16
+    h = _rand(n, d, seed=1)
+    hb = h.to(torch.bfloat16)
+    router = _rand(e, d, scale=0.05, seed=2)
+    w_gu, w_dn = _rand(e, 2 * f, d, scale=0.05, seed=3).to(torch.bfloat16), _rand(e, d, f, scale=0.05, seed=4).to(torch.bfloat16)
+    shared = (_rand(2 * f, d, scale=0.05, seed=5).to(torch.bfloat16), _rand(d, f, scale=0.05, seed=6).to(torch.bfloat16))
+    ids0, gates0, grouping0 = ops.moe_route(h, router, 1, group=True)
+    want = ops.materialize(ops.moe_experts(hb, ids0, gates0, w_gu, w_dn, shared_weights=shared, grouping=grouping0))
+    busy = _rand(2048, 2048, seed=7)
+    for _ in range(5):
+        busy @ busy  # (work on the first stream that the second must wait behind)
+        ids, gates, grouping = ops.moe_route(h, router, 1, group=True, beside=True)
+        assert (ops._route_done is not None) == (n >= ops.ROUTE_BESIDE_ROWS)
+        got = ops.materialize(ops.moe_experts(hb, ids, gates, w_gu, w_dn, shared_weights=shared, grouping=grouping))
+        assert ops._route_done is None
+        assert torch.equal(ids, ids0) and torch.equal(gates, gates0) and torch.equal(got, want)
+    ids, gates, _ = ops.moe_route(h, router, 1, group=True, beside=True)
+    ops.wait_route()  # (a caller that looks at the choice itself)
+    assert torch.equal(ids, ids0) and ops._route_done is None
+
+
 def test_moe_route_lowest_index_wins_ties(ops):
     h = _rand(5, 64, seed=1)
     w = _rand(1, 64, seed=2).expand(6, 64).contiguous()  # every expert the same score
