@@ -642,11 +642,11 @@ __global__ __launch_bounds__(WAVES * 64, DH <= 128 ? 2 : 1) void attention_prefi
 // (global_load_lds: a wavefront's 64 lanes fetch 16 bytes each from addresses of their own, and the kilobyte
 // lands in shared memory in lane order): no registers hold data on its way, nothing is stored to shared memory by
 // the wavefronts, and the only wait is for the loads asked for a step earlier.  What lands contiguously
-// decides the layout, and which piece a lane fetches makes it free of bank conflicts:
+// decides the layout (no padding is possible), and which piece a lane fetches spreads the reads over the banks:
 //   keys, per tile: [16 rows][16 pieces of 16 bytes], piece p of row r at place p ^ r: the 16 lanes that read
-//     the same piece of 16 different rows meet 16 different places;
+//     the same piece of 16 different rows read 16 different places of a row's 256 bytes;
 //   values, per tile: [128 elements][2 halves of 8 keys], half h of element d at place h ^ ((d >> 3) & 1): the 16
-//     lanes that read 8 bytes each of 16 consecutive elements meet 16 different pairs of banks.
+//     lanes that read 8 bytes each of 16 consecutive elements read 16 different 8-byte places of 256 bytes.
 // A step is 64 keys (four key tiles and four value tiles of 4 KB: each wavefront fetches the tile pair of its own
 // number), so that the maxima, the sums, the accumulators' correction, the barrier and the page look-up come once per
 // 64 keys; two buffers of 32 KB: a step's loads are asked for when the step before it begins, into the buffer that
