@@ -643,25 +643,35 @@ __global__ __launch_bounds__(WAVES * 64, DH <= 128 ? 2 : 1) void attention_prefi
 // lands in shared memory in lane order): no registers hold data on its way, nothing is stored to shared memory by
 // the wavefronts, and the only wait is for the loads asked for a step earlier.  What lands contiguously
 // decides the layout (no padding is possible), and which piece a lane fetches spreads the reads over the banks:
-//   keys, per tile: [16 rows][16 pieces of 16 bytes], piece p of row r at place p ^ r: the 16 lanes that read
-//     the same piece of 16 different rows read 16 different places of a row's 256 bytes;
-//   values, per tile: [128 elements][2 halves of 8 keys], half h of element d at place h ^ ((d >> 3) & 1): the 16
-//     lanes that read 8 bytes each of 16 consecutive elements read 16 different 8-byte places of 256 bytes.
+//   keys, per tile: [16 rows][16 pieces of 16 bytes], piece p of row r at place p ^ key_swizzle(r): eight
+//     neighbouring lanes that read the same piece of 8 different rows read 8 places that differ in their low three bits;
+//   values, per tile: [128 elements][2 halves of 8 keys], half h of element d at place h ^ ((d >> 2) & 1): eight
+//     neighbouring lanes that read the same half of 8 consecutive elements read 8 places that differ in their low
+//     three bits.  A lane reads a whole 16-byte piece (8 consecutive keys of one element) as its operand of the
+//     second product: the rows of the first product's key tiles are dealt so that a lane's eight probabilities
+//     belong to eight consecutive keys (see k_rd in the kernel).
 // A step is 64 keys (four key tiles and four value tiles of 4 KB: each wavefront fetches the tile pair of its own
 // number), so that the maxima, the sums, the accumulators' correction, the barrier and the page look-up come once per
 // 64 keys; two buffers of 32 KB: a step's loads are asked for when the step before it begins, into the buffer that
 // every wavefront has just left.  Measured at head size 128 against the kernel above (32 keys a step, through
-// registers): 15 % faster at 2,048 tokens, 20 % at 8,192; with 32 keys a step and the same loads it was 5 to 11 %.
+// registers): 15 % faster at 2,048 tokens, 20 % at 8,192; with 32 keys a step and the same loads it was 5 to 11 %;
+// the values as one 16-byte read per element instead of two of 8 bytes: another 10 to 17 %.
+// where piece p of key row r of a page tile lies: p ^ key_swizzle(r); the eight rows that eight neighbouring lanes read
+// (r % 4, r / 8 varying) then differ in the low three bits
+__device__ __forceinline__ int key_swizzle(int r) { return (r & 3) | ((r >> 3) << 2) | (((r >> 2) & 1) << 3); }
+
 __device__ __forceinline__ void load_to_lds16(const void* base, uint32_t byte_off, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n" ::"v"(byte_off), "s"(base), "s"(lds_addr) : "memory");
 }
 
 // One step of 64 keys (four tiles of 16) for the columns of a wavefront: softmax_and_values for twice the keys, so
-// that the maxima, the sums and the accumulators' correction are done once per 64 keys.  The values are taken from
-// shared memory half by half (tiles 0 and 1, then 2 and 3): sv points at the step's value tiles, v_rd is the lane's
-// offset in a tile, tile_bytes the distance between tiles.  halves: 1 if tiles 2 and 3 hold nothing for this wavefront.
+// that the maxima, the sums and the accumulators' correction are done once per 64 keys.  st[ct][2 h + t][i]: the
+// score of key 32 h + 8 g + 4 t + i of the step (g: the lane's group of 16), so the lane's eight probabilities of a
+// half h are those of keys 8 g .. 8 g + 7, and the values are read half by half as one 16-byte piece per element
+// (sv points at the step's value tiles, v_rd is the lane's offset in a tile, tile_bytes the distance between
+// tiles).  halves: 1 if the second half holds nothing for this wavefront.
 template <int DH, int CT, bool MASKED>
-__device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], const bool (&act)[4], int halves,
+__device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], int halves,
                                                      const unsigned char* sv, uint32_t v_rd, int tile_bytes, int kb,
                                                      const Columns (&col)[CT], int k_lo, int k_hi, float scale_log2,
                                                      float (&m)[CT], float (&l)[CT], f32x4 (&acc)[CT][DH / 16]) {
@@ -679,8 +689,8 @@ __device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], const b
       for (int i = 0; i < 4; ++i) {
         float v = st[ct][tt][i];
         if (MASKED) {
-          const int key = kb + 16 * tt + 4 * g + i;
-          const bool ok = act[tt] && key >= col[ct].lo && key <= col[ct].hi;
+          const int key = kb + 32 * (tt >> 1) + 8 * g + 4 * (tt & 1) + i;
+          const bool ok = key >= col[ct].lo && key <= col[ct].hi;
           v = ok ? v : -INFINITY;
           st[ct][tt][i] = v;
         }
@@ -723,9 +733,7 @@ __device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], const b
     uint4 vraw[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      const uint2 t0 = *reinterpret_cast<const uint2*>(sv + (2 * hf) * tile_bytes + v_rd + dt * 512);
-      const uint2 t1 = *reinterpret_cast<const uint2*>(sv + (2 * hf + 1) * tile_bytes + v_rd + dt * 512);
-      vraw[dt] = uint4{t0.x, t0.y, t1.x, t1.y};
+      vraw[dt] = *reinterpret_cast<const uint4*>(sv + (2 * hf + (g >> 1)) * tile_bytes + v_rd + dt * 512);
     }
     if (MASKED) {
       // values: keys outside [k_lo, k_hi] may never have been written: they are read as zero
@@ -734,7 +742,7 @@ __device__ __forceinline__ void softmax64_and_values(f32x4 (&st)[CT][4], const b
       for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
-          const int key = kb + 16 * (2 * hf + t2) + 4 * g + 2 * h2;
+          const int key = kb + 32 * hf + 8 * g + 4 * t2 + 2 * h2;
           const uint32_t lo_ok = (key >= k_lo && key <= k_hi) ? 0x0000ffffu : 0u;
           const uint32_t hi_ok = (key + 1 >= k_lo && key + 1 <= k_hi) ? 0xffff0000u : 0u;
           keep[t2][h2] = lo_ok | hi_ok;
@@ -827,17 +835,25 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = 4 * i + (lane >> 4);
-    const int piece = (lane & 15) ^ row;
+    const int piece = (lane & 15) ^ key_swizzle(row);
     k_src[i] = (uint32_t)(row * DH + piece * 8) * 2;
     const int d = 32 * i + (lane >> 1);
-    const int hh = (lane & 1) ^ ((d >> 3) & 1);
+    const int hh = (lane & 1) ^ ((d >> 2) & 1);
     v_src[i] = (uint32_t)(d * ps + hh * 8) * 2;
   }
   // what it reads: keys of tile tt, piece c * 4 + g of row c16; values of tile tt, keys 4 g .. 4 g + 3 of element d
-  uint32_t k_rd[KC];
+  // row r of the product's key tile t of a 32-key half is key 8 (r / 4) + 4 t + r % 4 of the half: a lane's eight
+  // probabilities then belong to eight consecutive keys (8 g .. 8 g + 7), whose values of one element are one 16-byte
+  // piece of the page; such a tile takes its rows from two tiles of the page (r / 8)
+  uint32_t k_rd[2][KC];
 #pragma unroll
-  for (int c = 0; c < KC; ++c) k_rd[c] = (uint32_t)(c16 * 256 + (((c * 4 + g) ^ c16) * 16));
-  const uint32_t v_rd = (uint32_t)((c16 * 2 + ((g >> 1) ^ (c16 >> 3))) * 16 + (g & 1) * 8);  // + dt * 512
+  for (int t = 0; t < 2; ++t) {
+    const int row = 8 * ((c16 >> 2) & 1) + 4 * t + (c16 & 3);
+#pragma unroll
+    for (int c = 0; c < KC; ++c)
+      k_rd[t][c] = (uint32_t)((c16 >> 3) * TILE + row * 256 + (((c * 4 + g) ^ key_swizzle(row)) * 16));
+  }
+  const uint32_t v_rd = (uint32_t)(c16 * 32 + (((g & 1) ^ ((c16 >> 2) & 1)) * 16));  // + dt * 512 + the page tile's
 
   bool bad = false;
   const int kb_first = (k_lo / 64) * 64;
@@ -893,22 +909,17 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
         if (tt >= 2 * halves) continue;
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
-          const uint4 kvv = *reinterpret_cast<const uint4*>(sb + tt * TILE + k_rd[c]);
+          const uint4 kvv = *reinterpret_cast<const uint4*>(sb + (tt >> 1) * (2 * TILE) + k_rd[tt & 1][c]);
           const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
 #pragma unroll
           for (int ct = 0; ct < CT; ++ct)
             st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
         }
       }
-      if (kb >= all_lo && kb + 63 <= all_hi) {  // the same for the whole wavefront
-        const bool act[4] = {true, true, true, true};
-        softmax64_and_values<DH, CT, false>(st, act, 2, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
-      } else {
-        bool act[4];
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) act[tt] = tt < 2 * halves && kb + 16 * tt <= k_hi && kb + 16 * tt + 15 >= k_lo;
-        softmax64_and_values<DH, CT, true>(st, act, halves, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
-      }
+      if (kb >= all_lo && kb + 63 <= all_hi)  // the same for the whole wavefront
+        softmax64_and_values<DH, CT, false>(st, 2, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
+      else  // (keys outside a column's range, those of tiles that were not asked for among them, count for nothing)
+        softmax64_and_values<DH, CT, true>(st, halves, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
     }
     buf ^= 1;
   }
