@@ -654,8 +654,9 @@ __global__ __launch_bounds__(WAVES * 64, DH <= 128 ? 2 : 1) void attention_prefi
 // number), so that the maxima, the sums, the accumulators' correction, the barrier and the page look-up come once per
 // 64 keys; two buffers of 32 KB: a step's loads are asked for when the step before it begins, into the buffer that
 // every wavefront has just left.  Measured at head size 128 against the kernel above (32 keys a step, through
-// registers): 15 % faster at 2,048 tokens, 20 % at 8,192; with 32 keys a step and the same loads it was 5 to 11 %;
-// the values as one 16-byte read per element instead of two of 8 bytes: another 10 to 17 %.
+// registers), the variants taking turns call by call: 26 % faster at 2,048 tokens, 24 % at 8,192 and 16,384; of that
+// 3 % are the loads (32 keys a step, three steps ahead), 14 % the 64 keys a step, 7 to 12 % the values as one 16-byte
+// read per element and the keys of a half asked for at once.
 // where piece p of key row r of a page tile lies: p ^ key_swizzle(r); the eight rows that eight neighbouring lanes read
 // (r % 4, r / 8 varying) then differ in the low three bits
 __device__ __forceinline__ int key_swizzle(int r) { return (r & 3) | ((r >> 3) << 2) | (((r >> 2) & 1) << 3); }
@@ -903,18 +904,28 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_lds_kernel(
       const int halves = kb + 32 <= my_hi ? 2 : 1;  // (tiles 2 and 3 lie past this wavefront's last key)
       f32x4 st[CT][4];
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
+      for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) st[ct][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (tt >= 2 * halves) continue;
 #pragma unroll
-        for (int c = 0; c < KC; ++c) {
-          const uint4 kvv = *reinterpret_cast<const uint4*>(sb + (tt >> 1) * (2 * TILE) + k_rd[tt & 1][c]);
-          const bf16x8 a = __builtin_bit_cast(bf16x8, kvv);
+      for (int hf = 0; hf < 2; ++hf) {
+        if (hf >= halves) break;
+        // a half's eight key pieces are asked for at once: one trip to shared memory, not one per pair of pieces, as the
+        // compiler orders them by itself (7 % of the kernel at 8,192 tokens)
+        bf16x8 kt[2][KC];
 #pragma unroll
-          for (int ct = 0; ct < CT; ++ct)
-            st[ct][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qb[ct][c], st[ct][tt], 0, 0, 0);
-        }
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int c = 0; c < KC; ++c)
+            kt[t][c] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(sb + hf * (2 * TILE) + k_rd[t][c]));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int c = 0; c < KC; ++c)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+              st[ct][2 * hf + t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kt[t][c], qb[ct][c], st[ct][2 * hf + t], 0, 0, 0);
       }
       if (kb >= all_lo && kb + 63 <= all_hi)  // the same for the whole wavefront
         softmax64_and_values<DH, CT, false>(st, 2, sb + 4 * TILE, v_rd, TILE, kb, col, k_lo, k_hi, scale_log2, m, l, acc);
