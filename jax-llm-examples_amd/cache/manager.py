@@ -62,6 +62,7 @@ class RequestEntry:
     reserved: int = 0  # tokens beyond num_tokens that have pages for the running step
     tables: list[list[int]] = dataclasses.field(default_factory=list)  # per group: page id or -1 per page index
     versions: list[int] = dataclasses.field(default_factory=list)  # per group: counts the changes of its table
+    serial: int = 0  # which life of which request this is: no two calls of add_request give the same
 
 
 @dataclasses.dataclass
@@ -192,6 +193,7 @@ class CacheManager:
         self.group_of: dict[int, int] = {}
         self.state: dict[int, torch.Tensor] = {}
         self.requests: dict[object, RequestEntry] = {}
+        self._lives = 0  # requests added so far
         item = torch.empty((), dtype=dtype).element_size()
         for key, cids in plan_groups(needs):
             (hk, dh), paged, retention = key
@@ -226,7 +228,9 @@ class CacheManager:
         slot = self.slots.alloc()
         for t in self.state.values():
             t[slot].zero_()
-        e = RequestEntry(slot=slot, tables=[[] for _ in self.groups], versions=[0 for _ in self.groups])
+        self._lives += 1
+        e = RequestEntry(slot=slot, tables=[[] for _ in self.groups], versions=[0 for _ in self.groups],
+                         serial=self._lives)
         self.requests[rid] = e
         return e
 
@@ -342,6 +346,15 @@ class CacheManager:
     def table_version(self, rid, group: int) -> int:
         """Changes whenever the request's block table of this group does (a copy kept elsewhere is then stale)."""
         return self.requests[rid].versions[group]
+
+    def table_stamp(self, rid) -> tuple:
+        """Equal stamps mean equal block tables: a copy of this request's tables kept elsewhere (a recorded
+        step's device buffer) is good as long as the stamp it was made under comes again.  The stamp names
+        this life of the request (a request that ended and was added again under the same id, as after a
+        preemption, has another: its version counts start again, its pages are others) and counts the
+        changes of every group's table."""
+        e = self.requests[rid]
+        return (e.serial, *e.versions)
 
     def num_free_pages(self) -> list[int]:
         return [g.pool.num_free for g in self.groups]

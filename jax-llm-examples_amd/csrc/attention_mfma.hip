@@ -1304,10 +1304,15 @@ __global__ __launch_bounds__(256, (CT == 1 && DH <= 128) ? 2 : 1) void attention
   if (alone) return;
 
   // ---- the last of the (token, kv head)'s blocks to get here merges the blocks' results
-  // They were written through to where every compute unit reads them (put_shared); once a thread's writes are
-  // done (the fence waits for them) and all threads have got there (the barrier), the ticket is taken, and the
-  // block that takes the last one reads the results from that same place (get_shared), not from a cache of its
-  // own die.  No cache is written back or emptied as a whole, as a fence over the whole GPU would do.
+  // What orders what: the results were written through to where every compute unit reads them (put_shared: a
+  // store that is acknowledged only when it has got there).  Every wavefront waits for the acknowledgement of
+  // all its outstanding stores (vmcnt(0): neither a workgroup-scope fence nor the barrier waits for them);
+  // then the barrier, so that all the block's stores are done before thread 0 takes the ticket; the ticket is
+  // an atomic at agent scope.  The block that takes the last ticket has thereby seen every other block's
+  // ticket, each taken after that block's stores were done; it reads the results with loads that go past its
+  // own die's caches (get_shared), issued after the ticket's value has come back.  No cache is written back
+  // or emptied as a whole, as a fence over the whole GPU would do.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (threadIdx.x == 0) {

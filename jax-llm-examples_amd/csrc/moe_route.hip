@@ -315,9 +315,13 @@ __global__ __launch_bounds__(256) void norm_route_kernel(const float* __restrict
     const float val = wave_sum(acc);
     if (lane == 0) put_shared(logits + n * E + e, val);
   }
-  // the last block to get here chooses and groups: the logits were written through to where every compute unit
-  // reads them; once a block's writes are done (the fence waits for them, the barrier for all its wavefronts)
-  // it takes a ticket
+  // the last block to get here chooses and groups.  The logits were written through to where every compute unit
+  // reads them (put_shared: a store acknowledged only when it has got there); every wavefront waits for the
+  // acknowledgement of its outstanding stores (vmcnt(0): neither the workgroup-scope fence nor the barrier
+  // does), the barrier for all the block's wavefronts, and only then the block takes its ticket (an atomic at
+  // agent scope).  The block with the last ticket reads the logits past its own die's caches (get_shared),
+  // after the ticket's value has come back.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (threadIdx.x == 0) {

@@ -22,79 +22,37 @@ from typing import Sequence
 import numpy as np
 import torch
 
-from .batch import GroupContext, StepContext, StepEntry, decode_bucket
+from .batch import StepEntry, StepLayout, context_over, decode_bucket, fill_step
 
 
 class _Recording:
     """One (number of requests, context bound) pair: its buffers, its context, its graph."""
 
     def __init__(self, model, cache, ops, num_requests: int, bucket: int) -> None:
-        R, ps = num_requests, cache.page_size
-        dev = model.device
+        R = num_requests
         self.R, self.bucket = R, bucket
-        self.width = -(-bucket // ps)
-        W = self.width
-        sizes = [("token_ids", R), ("positions", R), ("token_segment", R), ("cu_seqlens", R + 1),
-                 ("context_lens", R), ("state_slots", R), ("logits_indices", R)]
-        for g in cache.groups:
-            sizes += [(f"bt{g.index}", R * W), (f"sm{g.index}", R)]
-        total = sum(n for _, n in sizes)
+        width = -(-bucket // cache.page_size)
+        self.layout = StepLayout(R, R, R, [width] * len(cache.groups))
+        total = self.layout.size
         self.mirror = np.zeros(total, np.int32)  # what the device buffer shall hold, kept from step to step
-        self.views, o = {}, 0
-        for name, n in sizes:
-            self.views[name] = (o, o + n)
-            o += n
-        self.host = lambda name: self.mirror[self.views[name][0]: self.views[name][1]]
-        self.host("token_segment")[:] = np.arange(R)
-        self.host("cu_seqlens")[:] = np.arange(R + 1)
-        self.host("logits_indices")[:] = np.arange(R)
         for g in cache.groups:
-            self.host(f"bt{g.index}")[:] = -1
+            self.layout.view(self.mirror, f"block_table{g.index}")[:] = -1
+        self.stamps = [None] * R  # per row: the stamp of the block tables it holds (see fill_step)
         # two pinned staging buffers: the copy of one step may still be on its way when the next is laid out
         self.staging = [torch.empty(total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self.staged = [None, None]  # the event after each buffer's last copy
         self.turn = 0
-        self.device_buf = torch.zeros(total, dtype=torch.int32, device=dev)
-        d = lambda name: self.device_buf[self.views[name][0]: self.views[name][1]]
-        groups = []
-        for g in cache.groups:
-            groups.append(GroupContext(block_table=d(f"bt{g.index}").view(R, W), slot_mapping=d(f"sm{g.index}"),
-                                       width=W, retention=g.retention, seg_lens=[1] * R, seg_starts=None,
-                                       decode_bucket=bucket))
-        self.ctx = StepContext(
-            ops=ops, dtype=model.dtype, device=dev, num_tokens=R, num_segments=R, token_ids=d("token_ids"),
-            positions=d("positions"), token_segment=d("token_segment"), cu_seqlens=d("cu_seqlens"),
-            context_lens=d("context_lens"), state_slots=d("state_slots"), logits_indices=d("logits_indices"),
-            groups=groups, seg_lens=[1] * R, seg_starts=None, max_seg_len=1, max_context_len=bucket, page_size=ps)
-        self.rows = [None] * R  # per row: (request, its table versions) as last laid out
+        self.device_buf = torch.zeros(total, dtype=torch.int32, device=model.device)
+        self.ctx = context_over(self.layout, self.device_buf, cache, ops, model.dtype, model.device,
+                                seg_lens=[1] * R, seg_starts=None, max_context_len=bucket, bucket=bucket)
         self.graph = None
         self.logits = None
 
     def lay_out(self, cache, entries: Sequence[StepEntry], vocab_size: int) -> None:
-        """This step's numbers into the mirror, then one copy to the device."""
-        ps, W = cache.page_size, self.width
-        tok, pos = self.host("token_ids"), self.host("positions")
-        ctx_lens, slots = self.host("context_lens"), self.host("state_slots")
-        for i, e in enumerate(entries):
-            t = int(e.tokens[0])
-            if not 0 <= t < vocab_size:
-                raise ValueError(f"request {e.rid!r}: token id outside 0..{vocab_size - 1}")
-            req = cache.requests[e.rid]
-            p = req.num_tokens
-            tok[i], pos[i], ctx_lens[i], slots[i] = t, p, p + 1, req.slot
-            stamp = (e.rid, tuple(req.versions))
-            fresh = self.rows[i] != stamp
-            for g in cache.groups:
-                table = req.tables[g.index]
-                if fresh:
-                    row = self.host(f"bt{g.index}")[i * W: (i + 1) * W]
-                    row[: len(table)] = table
-                    row[len(table):] = -1
-                page = table[p // ps]
-                if page < 0:
-                    raise AssertionError(f"request {e.rid!r}: a new token has no page in group {g.index}")
-                self.host(f"sm{g.index}")[i] = page * ps + p % ps
-            self.rows[i] = stamp
+        """This step's numbers into the mirror (every row's logits are computed; the caller picks the wanted
+        ones), then one copy to the device."""
+        fill_step(self.layout, self.mirror, cache, [StepEntry(e.rid, e.tokens, (0,)) for e in entries], vocab_size,
+                  stamps=self.stamps)
         b = self.turn
         self.turn ^= 1
         if self.staged[b] is not None:

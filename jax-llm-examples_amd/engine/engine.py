@@ -22,20 +22,25 @@ from .scheduler import Request, Scheduler, SchedulerConfig
 
 
 class Engine:
+    DEFAULT_KV_MEMORY_FRACTION = 0.9
+
     def __init__(self, model, *, cache_tokens: Optional[int] = None, kv_memory_fraction: Optional[float] = None,
                  page_size: int = 16, decode_batch_size: int = 64, max_num_batched_tokens: int = 2048,
                  max_seq_len: Optional[int] = None, keep_free_pages: int = 0, reference_ops: bool = False,
                  poison: bool = False, decode_graphs: Optional[bool] = None) -> None:
         """The page pools are sized either by ``cache_tokens`` (tokens that a layer group which keeps
-        every token can hold; default ``decode_batch_size * max_seq_len``) or by ``kv_memory_fraction``
-        (that part of the device memory free now, after the weights).  Groups whose retention rule
+        every token can hold) or by ``kv_memory_fraction`` (that part of the device memory free now,
+        after the weights).  With neither: ``decode_batch_size * max_seq_len`` tokens if ``max_seq_len``
+        is given, else (on a GPU) 0.9 of the free memory.  Groups whose retention rule
         lets go of old tokens (chunked attention) get only what ``decode_batch_size`` requests can
         hold of them.  ``max_seq_len``: a request ends with reason ``"length"`` when prompt and
         output reach it; default: the configuration's ``max_position_embeddings``, if it has one.
         ``decode_graphs``: replay steps of single tokens as recorded HIP graphs (default: on a GPU)."""
         self.model = model
+        self.max_num_batched_tokens = max_num_batched_tokens
         self.ops = get_ops(model.device, reference_ops=reference_ops)
         limit = getattr(getattr(model, "config", None), "max_position_embeddings", None)
+        asked_len = max_seq_len
         if max_seq_len is None:
             max_seq_len = limit
         elif limit is not None and max_seq_len > limit:
@@ -52,9 +57,14 @@ class Engine:
             free, _ = torch.cuda.mem_get_info(model.device)
             memory = int(free * kv_memory_fraction)
         elif cache_tokens is None:
-            if max_seq_len is None:
+            if asked_len is not None:
+                cache_tokens = decode_batch_size * asked_len
+            elif model.device.type == "cuda":
+                # (the configuration's own limit may be millions of positions: take what the device has)
+                free, _ = torch.cuda.mem_get_info(model.device)
+                memory = int(free * self.DEFAULT_KV_MEMORY_FRACTION)
+            else:
                 raise ValueError("give cache_tokens, kv_memory_fraction or max_seq_len")
-            cache_tokens = decode_batch_size * max_seq_len
         num_pages = pool_sizes(needs, page_size=page_size, itemsize=item, max_requests=decode_batch_size,
                                max_step_tokens=max_num_batched_tokens, max_seq_len=max_seq_len,
                                cache_tokens=cache_tokens, memory_bytes=memory)
@@ -100,11 +110,35 @@ class Engine:
 
     # ------------------------------------------------------------------ the reference's two calls
     def prefill(self, tokens: Sequence[Sequence[int]], ids: Optional[Sequence] = None):
-        """Whole prompts in one step.  Returns ``(next_tokens, logits, ids)``: the greedy
-        next token of every prompt, the float32 logits at each prompt's last token, and
-        the handles to pass to :meth:`decode_step` (``model.py:1243-1267``)."""
+        """Whole prompts.  Returns ``(next_tokens, logits, ids)``: the greedy next token of every prompt, the
+        float32 logits at each prompt's last token, and the handles to pass to :meth:`decode_step`
+        (``model.py:1243-1267``).  Prompts that together fit the step's token budget
+        (``max_num_batched_tokens``) are one step; longer ones are run in portions of at most that many
+        tokens, which is what the page pools of layers that let go of old tokens are sized for."""
         ids = list(ids) if ids is not None else [f"req{next(self._ids)}" for _ in tokens]
-        logits = self.runner.step([StepEntry(i, list(t), [len(t) - 1]) for i, t in zip(ids, tokens)])
+        prompts = [list(t) for t in tokens]
+        if any(len(t) < 1 for t in prompts):
+            raise ValueError("a prompt needs at least one token")
+        done = [0] * len(prompts)
+        rows: dict = {}
+        while any(d < len(t) for d, t in zip(done, prompts)):
+            left, entries, closing = self.max_num_batched_tokens, [], []
+            for j, t in enumerate(prompts):
+                n = min(len(t) - done[j], left)
+                if n < 1:
+                    continue
+                last = done[j] + n == len(t)
+                entries.append(StepEntry(ids[j], t[done[j]: done[j] + n], [n - 1] if last else []))
+                if last:
+                    closing.append(j)
+                done[j] += n
+                left -= n
+            logits = self.runner.step(entries)
+            # (a step of single tokens hands out a buffer that the next such step writes again: what is kept
+            # and handed on is a copy)
+            for r, j in enumerate(closing):
+                rows[j] = logits[r].clone()
+        logits = torch.stack([rows[j] for j in range(len(prompts))])
         return self._greedy(logits), logits, ids
 
     def decode_step(self, last_tokens: Sequence[int], ids: Sequence):

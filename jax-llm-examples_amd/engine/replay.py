@@ -74,11 +74,14 @@ def main(argv=None) -> int:
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--max-requests", type=int, default=8, help="requests that may be live at once")
+    ap.add_argument("--poison", action="store_true",
+                    help="fill the page pools with NaN, and every page again when it is given back: a page that is "
+                         "read without having been written by its present holder then shows in the logits")
     ap.add_argument("--no-decode-graphs", action="store_true",
                     help="run steps of single tokens launch by launch instead of replaying recorded HIP graphs")
     args = ap.parse_args(argv)
     runner = make_runner(args.model, args.dtype, args.max_tokens, args.device, args.page_size, args.max_requests,
-                         decode_graphs=False if args.no_decode_graphs else None)
+                         poison=args.poison, decode_graphs=False if args.no_decode_graphs else None)
     replay(runner, sys.stdin, args.out)
     return 0
 

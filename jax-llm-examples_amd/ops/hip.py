@@ -133,8 +133,6 @@ class HipOps:
         # counters of the kernels in which the last wavefront (or block) to finish does the closing work: zero
         # between launches (whoever closes puts its counter back), so they are cleared here once
         self._tickets = torch.zeros(self.TICKETS, dtype=torch.int32, device=self.device)
-        self._side = None        # a second stream (default priority), made when first wanted
-        self._route_done = None  # the event behind a routing that runs on it (see moe_route)
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
         torch.set_float32_matmul_precision("highest")
@@ -603,30 +601,11 @@ class HipOps:
         return out
 
     # ------------------------------------------------------------------ routed experts
-    ROUTE_BESIDE_ROWS = 512  # from so many tokens on a routing asked for with ``beside`` runs on the second stream
-
-    def moe_route(self, h32, router, top_k: int, want_logits: bool = False, group: bool = False, beside: bool = False):
+    def moe_route(self, h32, router, top_k: int, want_logits: bool = False, group: bool = False):
         """``group``: also return the grouping of the choices by expert (what ``moe_align`` gives), made in
-        the same call; ``moe_experts`` takes it as ``grouping``.  ``beside``: the caller will hand the results to
-        ``moe_experts`` (or call ``wait_route`` before it looks at them): in a step of many tokens the router's
-        three small launches then run on a second stream, beside the shared expert's products that ``moe_experts``
-        starts with, and ``moe_experts`` waits for them before the routed experts' products."""
+        the same call; ``moe_experts`` takes it as ``grouping``."""
         n, d = h32.shape
         e = router.shape[0]
-        if (beside and group and not want_logits and n >= self.ROUTE_BESIDE_ROWS and not isinstance(h32, PendingNorm)
-                and not torch.cuda.is_current_stream_capturing()):
-            if self._side is None:
-                self._side = torch.cuda.Stream(device=self.device)
-            main = torch.cuda.current_stream(self.device)
-            self._side.wait_stream(main)
-            with torch.cuda.stream(self._side):
-                out = self.moe_route(h32, router, top_k, group=True)
-                self._route_done = torch.cuda.Event()
-                self._route_done.record(self._side)
-            for t in (out[0], out[1], *out[2]):
-                t.record_stream(main)
-            h32.record_stream(self._side)
-            return out
         if isinstance(h32, PendingNorm):
             fused = None if h32.done or not group else self._norm_route(h32, router, top_k)
             if fused is not None:
@@ -698,12 +677,6 @@ class HipOps:
         pending.x_out, pending.h = x_out, h
         return ids, gates, logits, (offsets, sorted_token, sorted_gate, inv)
 
-    def wait_route(self) -> None:
-        """The current stream waits for a routing that ``moe_route`` started beside it (nothing to do otherwise)."""
-        if self._route_done is not None:
-            torch.cuda.current_stream(self.device).wait_event(self._route_done)
-            self._route_done = None
-
     def moe_align(self, expert_ids, gates, num_experts: int, extra_group: bool = False):
         """Stable grouping of the (token, choice) pairs by expert: offsets ``[E + 1]``, the token and the gate of
         every sorted row, and where each pair went.  ``extra_group``: one more group behind the experts' that
@@ -737,7 +710,6 @@ class HipOps:
                 and m <= 2 * self.SKINNY_MAX_ROWS and tuple(shared_weights[0].shape) == (f2, d)
                 and tuple(shared_weights[1].shape) == (d, f2 // 2))
         if grouping is None or (fuse and grouping[0].numel() != e + 2):
-            self.wait_route()
             grouping = self.moe_align(expert_ids.contiguous(), gates.contiguous(), e, extra_group=fuse)
         offsets, sorted_token, sorted_gate, inv = grouping
         if fuse:
@@ -747,7 +719,6 @@ class HipOps:
             return ExpertSum(both[:m], inv, k, both[m:], n, d)
         if shared is None and shared_weights is not None:
             shared = self.linear(self.swiglu_linear(h, shared_weights[0]), shared_weights[1])
-        self.wait_route()
         if grouping[0].numel() != e + 1:  # (made with the extra group: the kernels below do not know of it)
             offsets, sorted_token, sorted_gate = offsets[: e + 1], sorted_token[:m], sorted_gate[:m]
         if mfma and m <= 2 * self.SKINNY_MAX_ROWS:  # few rows: the cost is streaming the chosen experts' weights

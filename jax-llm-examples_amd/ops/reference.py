@@ -168,10 +168,7 @@ class ReferenceOps:
         return out
 
     # ------------------------------------------------------------------ routed experts
-    def wait_route(self) -> None:
-        """(These ops run everything on one stream.)"""
-
-    def moe_route(self, h32, router, top_k: int, group: bool = False, beside: bool = False):
+    def moe_route(self, h32, router, top_k: int, group: bool = False):
         """Router logits in float32, the ``top_k`` largest per token (lowest index
         first among equals), gate = sigmoid of the chosen logit.  ``group``: a third result, the
         grouping of the choices by expert for ``moe_experts`` (none here: these ops do not group)."""

@@ -93,11 +93,9 @@ class MoESigmoidShared(FeedForward):
 
     def forward(self, h: torch.Tensor, h32: Optional[torch.Tensor], ctx) -> torch.Tensor:
         ops = ctx.ops
-        # (the results go to moe_experts, which starts with the shared expert: the kernel set may run the two side by side)
-        expert_ids, gates, grouping = ops.moe_route(h32, self.params["router"], self.top_k, group=True, beside=True)
+        expert_ids, gates, grouping = ops.moe_route(h32, self.params["router"], self.top_k, group=True)
         tap = getattr(ctx, "tap", None)
         if tap is not None:  # whoever watches the step sees the choice and may replace it
-            ops.wait_route()
             replaced = tap(self, "routing", (expert_ids, gates))
             if replaced is not None:
                 expert_ids, gates = replaced

@@ -47,3 +47,11 @@ def wide_model_dir_f32(tmp_path_factory):
     from tiny_configs import write_tiny
 
     return write_tiny("W", str(tmp_path_factory.mktemp("models_wide_f32") / "W"), torch.float32)
+
+
+@pytest.fixture(scope="session")
+def many_experts_model_dir_f32(tmp_path_factory):
+    """128 experts on the second of two layers at serving widths, in float32 (about 3.6 GB, written once)."""
+    from tiny_configs import write_tiny
+
+    return write_tiny("M", str(tmp_path_factory.mktemp("models_many_experts_f32") / "M"), torch.float32)

@@ -2,7 +2,7 @@
 function per part, float32 (or float64) throughout.
 
 It is written from the reference's formulas - each function cites the lines of
-``/root/reference/llama4/llama4_jax/model.py`` (``model.py`` below) it follows -
+``llama4/llama4_jax/model.py`` (``model.py`` below) it follows -
 and shares no code with the engine.  Where the task's configuration differs
 from what the reference hard-codes, the function says so:
 

@@ -18,7 +18,7 @@ from plain_llama4 import PlainModel
 from tiny_configs import FAST, TINY, write_tiny
 
 LENGTHS = {"A": [1, 80, 33, 47, 64, 9], "B": [120, 2, 49, 96, 31, 77], "C": [61, 40, 5, 83], "D": [37, 70, 3, 55, 64, 21],
-           "F": [300, 40, 170, 33], "W": [700, 33, 260, 48]}
+           "F": [300, 40, 170, 33], "W": [700, 33, 260, 48], "M": [2100, 33, 260, 48]}
 MODES = {"whole": traces.whole, "tail": traces.tail, "portions": traces.portions, "mixed": traces.mixed}
 TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}  # of the largest logit of the request
 
@@ -174,6 +174,45 @@ def test_gpu_bfloat16_serving_widths(wide_model_dir, mode):
     """Two layers (one rotary, one without) at the widths the benchmark runs: the kernel variants that only these
     sizes reach (rows of 5120, 40 heads on 8, experts 8192 wide) against the plain implementation."""
     _check("W", wide_model_dir, "bfloat16", "cuda:0", mode, reference_ops=False, plain_device="cuda:0")
+
+
+@pytest.fixture(scope="module")
+def many_experts_model_dir(tmp_path_factory):
+    return write_tiny("M", str(tmp_path_factory.mktemp("models_many_experts") / "M"), torch.bfloat16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(MODES))
+def test_gpu_bfloat16_many_experts_on_alternate_layers(many_experts_model_dir, mode):
+    """The larger model's shapes (``llama4/llama4_jax/configs.py:57-93``): a dense layer 16,384 wide, then a layer
+    of 128 experts (129 groups with the shared expert riding in their launches) at serving widths.  A prompt of
+    2,100 tokens gives every expert about 16 rows, some none; steps of a few tokens leave most experts empty."""
+    runner = make_runner(many_experts_model_dir, "bfloat16", 64, "cuda:0")
+    kinds = [type(b.feed_forward).__name__ for b in runner.model.blocks]
+    assert kinds == ["DenseSwiGLU", "MoESigmoidShared"] and runner.model.blocks[1].feed_forward.tiled
+    del runner
+    _check("M", many_experts_model_dir, "bfloat16", "cuda:0", mode, reference_ops=False, plain_device="cuda:0")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sixty_four_live_requests_with_many_experts(many_experts_model_dir, many_experts_model_dir_f32, dtype):
+    """64 live requests over 128 experts and a dense layer: steps of 64 single tokens (recorded in float32, where
+    the yardstick is the plain model in float64) beside portions of up to 300 tokens."""
+    folder = many_experts_model_dir if dtype == "bfloat16" else many_experts_model_dir_f32
+    g = torch.Generator().manual_seed(13)
+    lengths = torch.randint(60, 200, (64,), generator=g).tolist()
+    lengths[5] = 1100
+    mode = lambda reqs: traces.mixed(reqs, seed=4, max_live=64, decode_tail=16, max_portion=300)
+    _check("M", folder, dtype, "cuda:0", mode, reference_ops=False, plain_device="cuda:0",
+           record=dtype == "bfloat16", plain_dtype=torch.float64 if dtype == "float32" else torch.float32,
+           lengths=lengths, max_requests=64)
+
+
+@pytest.mark.gpu
+def test_gpu_float32_many_experts_mixed(many_experts_model_dir_f32):
+    _check("M", many_experts_model_dir_f32, "float32", "cuda:0", "mixed", reference_ops=False, plain_device="cuda:0",
+           plain_dtype=torch.float64, lengths=[700, 33, 260, 48, 48, 260, 33, 700])
 
 
 @pytest.mark.gpu

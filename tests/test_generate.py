@@ -95,6 +95,29 @@ def test_sampling_with_temperature_is_seeded_and_independent_of_the_batch(model_
     assert a == b and alone[0] == a[1] and a != greedy
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_prefill_of_a_prompt_longer_than_a_chunk_plus_a_steps_budget(model_dirs, device):
+    """The pools of layers that let go of old tokens hold a chunk plus one step's portion for every request: a
+    whole prompt beyond that is run in portions of the step's budget, and gives the same logits."""
+    plain = PlainModel(model_dirs["A"])  # chunk 32
+    g = torch.Generator().manual_seed(6)
+    long, short = (torch.randint(0, 512, (n,), generator=g).tolist() for n in (150, 9))
+    eng = _engine(model_dirs["A"], device, cache_tokens=176, decode_batch_size=2, max_num_batched_tokens=16)
+    chunked = [g_ for g_ in eng.cache.groups if g_.retention[0] == "chunk"]
+    assert chunked and all(g_.pool.num_pages * eng.cache.page_size < 150 for g_ in chunked)
+    nxt, logits, ids = eng.prefill([long, short])
+    steps = eng.runner.steps_run
+    assert steps == 10  # 159 tokens under a budget of 16
+    for row, toks, tok in zip(logits, (long, short), nxt):
+        ref = plain.logits(toks)[-1]
+        assert torch.allclose(row.cpu(), ref, rtol=1e-4, atol=2e-6) and tok == int(ref.argmax())
+    nxt2, l2 = eng.decode_step(nxt, ids)
+    ref = plain.logits(long + [nxt[0]])[-1]
+    assert torch.allclose(l2[0].cpu(), ref, rtol=1e-4, atol=2e-6)
+    eng.release(ids)
+    eng.cache.check()
+
+
 def test_engine_refuses_a_cpu_device_without_being_asked_for_the_plain_ops(model_dirs):
     with pytest.raises(RuntimeError, match="runs on a GPU"):
         Engine(load_model(model_dirs["A"], "float32", "cpu"), cache_tokens=64)
@@ -184,7 +207,7 @@ def test_trace_run_program(model_dirs_bf16, tmp_path, dtype):
     out_dir = tmp_path / "out"
     proc = subprocess.run(
         [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out",
-         str(out_dir), "--max-tokens", str(traces.max_live_tokens(steps))],
+         str(out_dir), "--max-tokens", str(traces.max_live_tokens(steps)), "--poison"],
         input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]

@@ -86,6 +86,20 @@ FAST["W"] = {
     "floor_scale": 8192, "attn_scale": 0.1, "rms_norm_eps": 1e-5, "tie_word_embeddings": False,
 }
 
+# The shapes of the larger Llama 4 (``llama4/llama4_jax/configs.py:57-93``: experts on every second layer, 128 of
+# them, dense layers 16,384 wide between, no frequency scaling) at serving widths, with the experts' width cut (not
+# their number) so that the plain model stays cheap: about 1.8 GB in bfloat16 (GPU tests only)
+FAST["M"] = {
+    "architectures": ["Llama4ForCausalLM"],
+    "seed": 79,
+    "num_hidden_layers": 2, "hidden_size": 5120, "num_attention_heads": 40, "num_key_value_heads": 8,
+    "head_dim": 128, "interleave_moe_layer_step": 2, "num_local_experts": 128, "num_experts_per_tok": 1,
+    "intermediate_size": 256, "intermediate_size_mlp": 16384, "vocab_size": 20008, "rope_theta": 500000.0,
+    "rope_scaling": None, "no_rope_layers": [1, 0], "attention_chunk_size": 8192, "use_qk_norm": True,
+    "attn_temperature_tuning": True, "floor_scale": 8192, "attn_scale": 0.1, "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False,
+}
+
 
 def tiny_config_json(name: str) -> dict:
     c = {k: v for k, v in {**TINY, **FAST}[name].items() if k != "seed"}
