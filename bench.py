@@ -5,7 +5,10 @@ one MI355X.
 
 prints one JSON line: ``value`` = decoded tokens per second at batch 8 and context 4,096
 (a "step" is one decode step of the whole batch, sampling included), plus the prefill of
-2,048 tokens, the decode step's HBM roofline fraction, and decode at batch 1 and 64.
+2,048 tokens, the decode step's HBM roofline fraction and, under ``points``, decode at other
+batch sizes and context lengths (``decode_b<batch>[_c<context>]``: tokens a second, with
+``..._hbm_frac``: the step's bytes / its time / 8 TB/s) and longer prefills
+(``prefill_<tokens>``: tokens a second, ``..._frac`` of the dtype's MFMA peak).
 """
 from __future__ import annotations
 
@@ -33,7 +36,9 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
+    ap.add_argument("--points", default="1,64,16,32,128@2048,8@16384,8@32768",
+                    help="other decode steps to report: batch or batch@context, comma-separated")
+    ap.add_argument("--prefill-points", default="8192", help="other prefill lengths to report")
     ap.add_argument("--point-steps", type=int, default=12)
     ap.add_argument("--preset", default="llama4-scout")
     ap.add_argument("--no-prefill", action="store_true")
@@ -64,8 +69,15 @@ def main() -> int:
           f"({model.num_parameters() / 1e9:.1f} B parameters)", file=sys.stderr, flush=True)
 
     page = 16
-    batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
-    need_tokens = max(batches) * (args.context + page) + args.prefill_tokens + 4 * page
+    points_at = []  # (batch, context)
+    for spec in args.points.split(","):
+        if spec:
+            b, _, c = spec.partition("@")
+            points_at.append((int(b), int(c) if c else args.context))
+    prefill_points = [] if args.no_prefill else [int(t) for t in args.prefill_points.split(",") if t]
+    batches = [args.batch] + [b for b, _ in points_at]
+    need_tokens = (max([args.batch * (args.context + page)] + [b * (c + page) for b, c in points_at])
+                   + max([args.prefill_tokens] + prefill_points) + 4 * page)
     ops = get_ops(dev)
     cache = CacheManager(model.cache_needs(), page_size=page, num_pages=-(-need_tokens // page),
                          max_requests=max(batches) + 1, dtype=model.dtype, device=dev)
@@ -82,29 +94,31 @@ def main() -> int:
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
 
     # ------------------------------------------------------------------ prefill of 2,048 tokens
-    prefill = None
-    if not args.no_prefill:
-        T = args.prefill_tokens
+    def run_prefill(T: int, tries: int):
         times = []
-        for it in range(3):
+        for it in range(tries):
             toks = torch.randint(0, V, (T,), generator=gen).tolist()
             torch.cuda.synchronize()
             t1 = time.perf_counter()
-            logits = runner.step([StepEntry(f"p{it}", toks, [T - 1])])
+            logits = runner.step([StepEntry(f"p{T}_{it}", toks, [T - 1])])
             sampler(logits, [greedy], [0])
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t1)
-            runner.finish(f"p{it}")
+            runner.finish(f"p{T}_{it}")
             print(f"[bench] prefill of {T} tokens: {times[-1] * 1e3:.1f} ms", file=sys.stderr, flush=True)
         sec = min(times[1:])
-        fl = prefill_flops(model, T)
-        prefill = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 2),
-                   "frac": round(fl / sec / PEAK_FLOPS[dkey], 4)}
+        return sec, prefill_flops(model, T) / sec / PEAK_FLOPS[dkey]
+
+    prefill = None
+    if not args.no_prefill:
+        T = args.prefill_tokens
+        sec, frac = run_prefill(T, 3)
+        prefill = {"value": round(T / sec, 1), "tokens": T, "ms": round(sec * 1e3, 2), "frac": round(frac, 4)}
 
     # ------------------------------------------------------------------ decode
-    def decode(batch: int, steps: int, warmup: int):
-        ctx0 = args.context - (steps + warmup)
-        ids = [f"d{batch}_{i}" for i in range(batch)]
+    def decode(batch: int, steps: int, warmup: int, context: int):
+        ctx0 = context - (steps + warmup)
+        ids = [f"d{batch}_{context}_{i}" for i in range(batch)]
         for rid in ids:  # contexts stand in: pages are taken, their contents are the random fill
             cache.add_request(rid)
             cache.reserve(rid, ctx0)
@@ -133,16 +147,22 @@ def main() -> int:
         nbytes = decode_step_bytes(model, cache, contexts, watcher)
         for rid in ids:
             runner.finish(rid)
-        print(f"[bench] decode batch {batch}: {sec * 1e3:.2f} ms/step, {batch / sec:.1f} tok/s, "
+        print(f"[bench] decode batch {batch} at context {context}: {sec * 1e3:.2f} ms/step, {batch / sec:.1f} tok/s, "
               f"{nbytes['total'] / 1e9:.1f} GB/step -> {nbytes['total'] / sec / 1e9:.0f} GB/s", file=sys.stderr,
               flush=True)
         return sec, nbytes, (sum(distinct.values()) / max(1, len(distinct)))
 
-    sec, nbytes, mean_experts = decode(args.batch, args.steps, args.warmup)
+    sec, nbytes, mean_experts = decode(args.batch, args.steps, args.warmup, args.context)
     points = {}
-    for b in batches[1:]:
-        s, _, _ = decode(b, args.point_steps, 2)
-        points[f"decode_b{b}"] = round(b / s, 1)
+    for b, c in points_at:
+        s_, nb, _ = decode(b, args.point_steps, 2, c)
+        key = f"decode_b{b}" + (f"_c{c}" if c != args.context else "")
+        points[key] = round(b / s_, 1)
+        points[key + "_hbm_frac"] = round(nb["total"] / s_ / 1e9 / PEAK_HBM_GBS, 4)
+    for T in prefill_points:
+        s_, frac = run_prefill(T, 2)
+        points[f"prefill_{T}"] = round(T / s_, 1)
+        points[f"prefill_{T}_frac"] = round(frac, 4)
 
     achieved = nbytes["total"] / sec / 1e9
     out = {

@@ -42,7 +42,8 @@ _SIGNATURES = {
     "jle_attention_decode_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _f, _i, _i,
                                    _i, _i, _vp, _f, _f, _f, _vp, _i, _vp],
     "jle_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
-    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _vp],
+    "jle_gemm_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _vp, _vp,
+                        _vp],
     "jle_gemm_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
 }
 
@@ -133,6 +134,8 @@ class HipOps:
         # counters of the kernels in which the last wavefront (or block) to finish does the closing work: zero
         # between launches (whoever closes puts its counter back), so they are cleared here once
         self._tickets = torch.zeros(self.TICKETS, dtype=torch.int32, device=self.device)
+        self._slice_tickets = torch.zeros(self.SLICE_TICKETS, dtype=torch.int32, device=self.device)
+        self._compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         torch.backends.cuda.matmul.allow_tf32 = False
         torch.backends.cudnn.allow_tf32 = False
         torch.set_float32_matmul_precision("highest")
@@ -269,11 +272,32 @@ class HipOps:
     SKINNY_LINEAR_ROWS = 8  # plain projections (q|k|v, o, down)
     SHARED_RIDES_ROWS = 16  # a shared expert's two products ride in the routed experts' launches as one more group
 
+    SLICE_TICKETS = 1 << 14
+    SLICE_ROWS = 16  # up to so many rows the row tiles of a launch may be cut along K (see _k_slices)
+    SLOT_ROWS = 16  # a grouped product of so few rows is launched over as many group slots as it has rows
+
+    def _k_slices(self, tiles: int) -> tuple:
+        """How a launch of ``tiles`` row tiles (a block each) is evened out over the compute units: ``(m, s)``
+        = the first ``m`` tiles cut into ``s`` slices along K, so that the blocks are a multiple of the compute
+        units; ``(0, 0)``: leave it (already even, or so many blocks that a part of a round does not matter)."""
+        cus = self._compute_units
+        m = tiles % cus
+        # (measured on 256 compute units: 320 tiles gain a tenth to a fifth, 448 tiles lose as much: three
+        # quarters of them would be cut)
+        if m == 0 or tiles > 0.8 * (-(-tiles // cus) * cus):
+            return 0, 0
+        for s in (2, 4, 8):
+            if (m * s) % cus == 0:
+                return m, s
+        return 0, 0
+
     def gemm_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,
-                    variant=0, tiled=False, b_last=None, tiled_last=False):
+                    variant=0, tiled=False, b_last=None, tiled_last=False, balance=True):
         """bfloat16 weight-streaming product on MFMA for few rows (see ``gemm_skinny.hip``); with ``swiglu`` the
         result is ``silu(gate) * up`` of the two halves of ``b``'s rows.  ``b_last``: one more group behind
-        ``b``'s, its matrix a tensor of its own (``offsets`` then has an entry more)."""
+        ``b``'s, its matrix a tensor of its own (``offsets`` then has an entry more).  ``balance``: with up to 16
+        rows, cut some row tiles along K so that the launch's blocks are a multiple of the compute units, and
+        launch a grouped product over as many group slots as it has rows (not over every group)."""
         if b.dim() == 2:
             b = b.unsqueeze(0)
         g, nout, k = b.shape
@@ -291,8 +315,21 @@ class HipOps:
             raise KernelError(f"the MFMA product needs an inner size that is a multiple of 8, got {k}")
         out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32 if out_f32 else torch.bfloat16,
                           device=a.device)
+        slots = split_tiles = split = 0
+        ws = None
+        if balance and m <= self.SLICE_ROWS and variant <= 0:
+            if offsets is not None and g > m and g <= 4096 and m <= self.SLOT_ROWS:
+                slots = m  # (no more groups have rows than there are rows)
+            if not swiglu and (offsets is None or slots):
+                split_tiles, split = self._k_slices(-(-nout // 16))
+                units = max(slots, 1) * split_tiles
+                if units > self.SLICE_TICKETS or (k + 63) // 64 < split:
+                    split_tiles = split = 0
+                elif split_tiles:
+                    ws = torch.empty(units * split * 256, dtype=torch.float32, device=a.device)
         self._call("jle_gemm_skinny", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu),
-                   int(out_f32), m, nout, k, g, m, variant, int(tiled), _p(b_last), int(tiled_last))
+                   int(out_f32), m, nout, k, g, m, variant, int(tiled), _p(b_last), int(tiled_last), slots,
+                   split_tiles, split, _p(ws), _p(self._slice_tickets))
         return out
 
     def gemm_grouped(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, out_f32=False, rows=None,

@@ -685,6 +685,62 @@ def test_weight_streaming_product(ops, ref, m, nout, k, out_f32):
     assert err <= (2e-5 if out_f32 else 5e-3), err  # float32 out: only the order of the sum differs
 
 
+@pytest.mark.parametrize("m", [1, 8, 16])
+@pytest.mark.parametrize("nout,k", [(5120, 320), (5120, 8192), (1024, 264), (9216, 5120), (2048, 512)])
+def test_weight_streaming_product_with_row_tiles_cut_along_k(ops, m, nout, k):
+    """Row tiles that do not fill a round of the compute units are cut along K, each slice a block of its own,
+    and the slices' sums are added by the tile's last block in the slices' order: the same bits every time, in
+    both layouts, and the tickets are back at zero."""
+    from jax_llm_examples_amd.ops.layout import can_tile, tile_
+    tiles = -(-nout // 16)
+    cut, slices = ops._k_slices(tiles)
+    assert cut > 0 and (cut * slices) % ops._compute_units == 0, "sizes chosen so that tiles are cut"
+    a, b = _rand(m, k, dt=torch.bfloat16, seed=1), _rand(nout, k, dt=torch.bfloat16, scale=0.1, seed=2)
+    want = a.float() @ b.float().t()
+    got = ops.gemm_skinny(a, b, out_f32=True)
+    assert float((got - want).abs().max() / want.abs().max()) <= 2e-5
+    whole = ops.gemm_skinny(a, b, out_f32=True, balance=False)  # (sums in another order: other blocks, other bits)
+    assert float((whole - want).abs().max() / want.abs().max()) <= 2e-5
+    for _ in range(3):
+        assert torch.equal(ops.gemm_skinny(a, b, out_f32=True), got)
+    if can_tile(b):
+        bt = b.clone()
+        tile_(bt)
+        assert torch.equal(ops.gemm_skinny(a, bt, out_f32=True, tiled=True), got)
+    assert int(ops._slice_tickets.abs().sum()) == 0
+
+
+@pytest.mark.parametrize("n,e,nout,k", [(1, 16, 5120, 512), (2, 128, 5120, 256), (8, 16, 5120, 8192), (7, 128, 320, 64),
+                                        (16, 40, 2048, 128)])
+def test_weight_streaming_product_over_group_slots(ops, n, e, nout, k):
+    """A grouped product of few rows is launched over as many group slots as it has rows (slot j: the j-th group
+    that has rows), with a last group whose matrix is a tensor of its own: the same result as over every group."""
+    dt = torch.bfloat16
+    g = torch.Generator().manual_seed(n)
+    ids = torch.randint(0, e, (n, 1), generator=g).to(torch.int32).to(DEV)
+    gates = torch.rand(n, 1, generator=g).to(DEV)
+    off, tok, gate, inv = ops.moe_align(ids, gates, e, extra_group=True)
+    x = _rand(2 * n, k, dt=dt, seed=1)  # (rows already grouped: the second product of an expert layer)
+    w, w_last = _rand(e, nout, k, dt=dt, scale=0.1, seed=2), _rand(nout, k, dt=dt, scale=0.1, seed=3)
+    got = ops.gemm_skinny(x, w, offsets=off, b_last=w_last, out_f32=True)
+    every = ops.gemm_skinny(x, w, offsets=off, b_last=w_last, out_f32=True, balance=False)
+    sorted_ids = ids.flatten()[tok[:n].long()].long()
+    want = torch.cat([torch.einsum("nk,nok->no", x[:n].float(), w[sorted_ids].float()),
+                      x[n:].float() @ w_last.float().t()])
+    assert float((got - want).abs().max() / want.abs().max()) <= 2e-5
+    assert float((every - want).abs().max() / want.abs().max()) <= 2e-5
+    if ops._k_slices(-(-nout // 16))[0] == 0:  # (no tile cut: the same blocks form the same sums)
+        assert torch.equal(got, every)
+    # gathered rows, scaled, with the fused activation (the first product of an expert layer)
+    h = _rand(n, k, dt=dt, seed=4)
+    wgu, wgu_last = _rand(e, 2 * 64, k, dt=dt, scale=0.1, seed=5), _rand(2 * 64, k, dt=dt, scale=0.1, seed=6)
+    a1 = ops.gemm_skinny(h, wgu, offsets=off, a_rows=tok, scale=gate, swiglu=True, b_last=wgu_last, rows=2 * n)
+    a2 = ops.gemm_skinny(h, wgu, offsets=off, a_rows=tok, scale=gate, swiglu=True, b_last=wgu_last, rows=2 * n,
+                         balance=False)
+    assert torch.equal(a1, a2)
+    assert int(ops._slice_tickets.abs().sum()) == 0
+
+
 @pytest.mark.parametrize("n,d,f,e,k", [(8, 128, 48, 16, 1), (64, 5120, 64, 16, 1), (20, 264, 40, 3, 2), (3, 64, 24, 128, 1)])
 def test_weight_streaming_product_grouped_with_swiglu(ops, ref, n, d, f, e, k):
     dt = torch.bfloat16
