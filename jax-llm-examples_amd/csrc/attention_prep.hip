@@ -162,7 +162,7 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(const T* __restrict
                                                              int Hkv, int dh, int page_size, int write_kv) {
   const int lane = threadIdx.x & 63;
   const int H = Hq + 2 * Hkv;
-  const int H_here = write_kv ? H : Hq;
+  const int H_here = write_kv == 1 ? H : write_kv == 2 ? Hq + Hkv : Hq;  // (2: the values are written by value_write_kernel)
   const int lph = dh >> 3;          // lanes per head
   const int hps = 64 / lph;         // heads per set
   const int per_wave = hps * ROUNDS;
@@ -241,6 +241,43 @@ __global__ __launch_bounds__(256) void qk_prepare_vec_kernel(const T* __restrict
   }
 }
 
+// The values of many tokens into their pages.  In a page one element of all its tokens is contiguous, so a token's
+// elements lie page_size apart: written token by token, every 2- or 4-byte store is a memory transaction of its
+// own.  Here a block takes 16 consecutive tokens of the step and one kv head, turns their values round in shared
+// memory and writes with the token as the fastest index: tokens that follow each other in a page (a segment's
+// do) fill whole 32- or 64-byte pieces.
+template <typename T>
+__global__ __launch_bounds__(256) void value_write_kernel(const T* __restrict__ qkv, T* __restrict__ kv_cache,
+                                                          const int* __restrict__ slot_mapping, int N, int Hq, int Hkv,
+                                                          int dh, int page_size) {
+  __shared__ __attribute__((aligned(16))) T tile[16][128 + 8];
+  __shared__ int slot_s[16];
+  const int t0 = blockIdx.x * 16, hk = blockIdx.y, t = threadIdx.x;
+  const int H = Hq + 2 * Hkv;
+  if (t < 16) slot_s[t] = t0 + t < N ? slot_mapping[t0 + t] : -1;
+  for (int d0 = 0; d0 < dh; d0 += 128) {
+    const int width = min(128, dh - d0);  // a multiple of 8
+    __syncthreads();
+    {
+      const int j = t >> 4, p = t & 15;  // token, piece of 8 elements
+      if (t0 + j < N && 8 * p < width) {
+        // (16-byte pieces: the rows of q|k|v and of the tile are aligned to them)
+        const uint4* src = reinterpret_cast<const uint4*>(qkv + ((size_t)(t0 + j) * H + Hq + Hkv + hk) * dh + d0 + 8 * p);
+        uint4* dst = reinterpret_cast<uint4*>(&tile[j][8 * p]);
+#pragma unroll
+        for (int i = 0; i < (int)(8 * sizeof(T) / 16); ++i) dst[i] = src[i];
+      }
+    }
+    __syncthreads();
+    const int j = t & 15;
+    const int slot = slot_s[j];
+    if (slot < 0) continue;
+    const int page = slot / page_size, off = slot - page * page_size;
+    T* plane = kv_cache + (((size_t)page * 2 + 1) * Hkv + hk) * page_size * dh + off;
+    for (int d = t >> 4; d < width; d += 16) plane[(size_t)(d0 + d) * page_size] = tile[j][d];
+  }
+}
+
 JLE_API int jle_qk_prepare(const void* qkv, void* q_out, void* kv_cache, const int* positions,
                            const int* slot_mapping, const float* inv_freq, float norm_eps, float floor_scale,
                            float attn_scale, int is_bf16, int N, int Hq, int Hkv, int dh, int page_size,
@@ -256,7 +293,20 @@ JLE_API int jle_qk_prepare(const void* qkv, void* q_out, void* kv_cache, const i
                      norm_wk == nullptr && !norm_first;
   const bool aligned = (((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)kv_cache) & 31) == 0;
   if (usual && aligned && dh >= 16 && dh <= 512 && (dh & (dh - 1)) == 0) {  // whatever N: a token's result is the same
-    const int H_here = write_kv ? Hq + 2 * Hkv : Hq;
+    // many tokens: their values go into the pages through a kernel of their own, sixteen tokens at a time
+    const bool values_apart = write_kv && N >= 64 && Hkv <= 65535;
+    if (values_apart) {
+      dim3 gw((N + 15) / 16, Hkv), bw(256);
+      if (is_bf16)
+        hipLaunchKernelGGL(value_write_kernel<bf16_t>, gw, bw, 0, s, (const bf16_t*)qkv, (bf16_t*)kv_cache,
+                           slot_mapping, N, Hq, Hkv, dh, page_size);
+      else
+        hipLaunchKernelGGL(value_write_kernel<float>, gw, bw, 0, s, (const float*)qkv, (float*)kv_cache,
+                           slot_mapping, N, Hq, Hkv, dh, page_size);
+      JLE_LAUNCH_CHECK();
+      write_kv = 2;
+    }
+    const int H_here = write_kv == 1 ? Hq + 2 * Hkv : write_kv == 2 ? Hq + Hkv : Hq;
     const int rounds = (long long)N * H_here >= 8192 ? 4 : 1;
     const int per_wave = (64 / (dh / 8)) * rounds;
     const long long waves = (long long)N * ((H_here + per_wave - 1) / per_wave);
