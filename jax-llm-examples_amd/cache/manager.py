@@ -25,7 +25,7 @@ from typing import Optional
 
 import torch
 
-from ..parts.base import CacheNeed, first_needed_position
+from ..parts.base import CacheNeed, first_needed_position, kept_prefix, retention_kind
 from .pages import OutOfPages, OutOfSlots, PagePool, SlotPool
 
 
@@ -63,6 +63,8 @@ class RequestEntry:
     tables: list[list[int]] = dataclasses.field(default_factory=list)  # per group: page id or -1 per page index
     versions: list[int] = dataclasses.field(default_factory=list)  # per group: counts the changes of its table
     serial: int = 0  # which life of which request this is: no two calls of add_request give the same
+    freed_upto: list[int] = dataclasses.field(default_factory=list)  # per group: pages below this index (and beyond
+    # the rule's kept prefix) have been given back
 
 
 @dataclasses.dataclass
@@ -108,10 +110,7 @@ def tokens_held_at_most(retention: tuple, max_step_tokens: int, max_seq_len: Opt
     """The most tokens of one request that a group with this retention rule holds at any time
     (``None``: no bound but the sequence's length): what the rule keeps for the next query plus the
     portion of the running step, whose pages are given back only after it."""
-    kind = retention[0]
-    cap = None
-    if kind in ("chunk", "window"):
-        cap = int(retention[1]) + max_step_tokens
+    cap = retention_kind(retention).held_at_most(retention, max_step_tokens)
     if max_seq_len is not None:
         cap = max_seq_len if cap is None else min(cap, max_seq_len)
     return cap
@@ -197,6 +196,7 @@ class CacheManager:
         item = torch.empty((), dtype=dtype).element_size()
         for key, cids in plan_groups(needs):
             (hk, dh), paged, retention = key
+            retention_kind(retention)  # (an unknown rule is an error here, not at the first page given back)
             i = len(self.groups)
             n = num_pages[i] if isinstance(num_pages, dict) else num_pages
             g = CacheGroup(i, hk, dh, retention, list(cids), PagePool(n), {}, paged=paged, itemsize=item)
@@ -230,7 +230,7 @@ class CacheManager:
             t[slot].zero_()
         self._lives += 1
         e = RequestEntry(slot=slot, tables=[[] for _ in self.groups], versions=[0 for _ in self.groups],
-                         serial=self._lives)
+                         serial=self._lives, freed_upto=[0 for _ in self.groups])
         self.requests[rid] = e
         return e
 
@@ -292,8 +292,11 @@ class CacheManager:
         for g in self.groups:
             keep_from = first_needed_position(g.retention, e.num_tokens)
             table = e.tables[g.index]
-            # page j holds positions [j*ps, (j+1)*ps): free iff (j+1)*ps <= keep_from
-            gone = [j for j in range(min(len(table), keep_from // self.page_size)) if table[j] >= 0]
+            # page j holds positions [j*ps, (j+1)*ps): free iff it lies wholly in [kept prefix, keep_from)
+            first = max(e.freed_upto[g.index], -(-kept_prefix(g.retention) // self.page_size))
+            upto = min(len(table), keep_from // self.page_size)
+            gone = [j for j in range(first, upto) if table[j] >= 0]
+            e.freed_upto[g.index] = max(e.freed_upto[g.index], upto)
             if gone:
                 self._release(g, [table[j] for j in gone])
                 e.versions[g.index] += 1

@@ -72,6 +72,9 @@ class ModelPlan:
     order: tuple[OrderEntry, ...]
     final_norm: PartSpec
     tie_word_embeddings: bool = False
+    # the model's two ends; None: a plain token table and a plain linear head (tied if tie_word_embeddings)
+    embedding: PartSpec | None = None
+    head: PartSpec | None = None
 
     def __post_init__(self) -> None:
         seen_write: dict[int, int] = {}

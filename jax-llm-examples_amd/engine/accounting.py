@@ -5,7 +5,7 @@ reports its own numbers (:meth:`~..parts.base.Part.step_weight_bytes`,
 here knows a kind of part."""
 from __future__ import annotations
 
-from ..parts.base import first_needed_position
+from ..parts.base import first_needed_position, kept_prefix
 
 
 def _nbytes(t) -> int:
@@ -34,13 +34,12 @@ def decode_step_bytes(model, cache, contexts, watcher: StepWatcher | None = None
             observed = next(iter(seen.values())) if seen else None
             weights += part.step_weight_bytes(observed)
     weights += model.final_norm.step_weight_bytes()
-    head = model.embed if model.lm_head is None else model.lm_head
-    weights += _nbytes(head.params["weight"])
-    weights += len(contexts) * model.plan.hidden_size * model.embed.params["weight"].element_size()
+    weights += model.lm_head.step_bytes(model.embed) + model.embed.step_bytes(len(contexts))
     kv = 0
     for g in cache.groups:
         for c in contexts:
-            visible = c - first_needed_position(g.retention, c - 1)
+            first = first_needed_position(g.retention, c - 1)
+            visible = c - first + min(first, kept_prefix(g.retention))
             kv += visible * g.bytes_per_token()
     return {"weights": weights, "kv": kv, "total": weights + kv}
 
@@ -54,5 +53,4 @@ def prefill_flops(model, num_tokens: int, start: int = 0) -> float:
         b = model.blocks[e.layer]
         per_token += sum(p.flops_per_token() for p in b.parts().values())
         mixing += b.mixer.mixing_flops(start, num_tokens)
-    head = model.embed if model.lm_head is None else model.lm_head
-    return per_token * num_tokens + 2.0 * head.params["weight"].numel() + mixing
+    return per_token * num_tokens + model.lm_head.flops_per_token() + mixing

@@ -77,7 +77,7 @@ class DecodeGraphs:
         self.captures = 0
         self.safe = (getattr(ops, "name", "") == "hip" and model.device.type == "cuda"
                      and all(getattr(p, "graph_safe", False) for b in model.blocks for p in b.parts().values())
-                     and getattr(model.final_norm, "graph_safe", False))
+                     and all(getattr(p, "graph_safe", False) for p in (model.final_norm, model.embed, model.lm_head)))
 
     def fits(self, entries: Sequence[StepEntry], tap) -> bool:
         return self.safe and tap is None and all(len(e.tokens) == 1 for e in entries)

@@ -13,7 +13,15 @@ import torch
 
 from . import build as _build
 
-_RET_MODES = {"all": 0, "chunk": 1, "window": 2}
+_RET_MODES = {"all": 0, "chunk": 1, "window": 2}  # the rules under which the attention kernels here read keys
+
+
+def _ret_mode(retention) -> int:
+    try:
+        return _RET_MODES[retention[0]]
+    except KeyError:
+        raise KernelError(f"the attention kernels read keys under the rules {', '.join(_RET_MODES)}; a mixer with the "
+                          f"rule {retention!r} brings kernels of its own") from None
 
 _vp, _i, _f, _ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_longlong
 
@@ -473,7 +481,7 @@ class HipOps:
             ws_o = torch.empty(units * dh, dtype=torch.float32, device=qkv.device)
             out = torch.empty(n, hq * dh, dtype=qkv.dtype, device=qkv.device)
             fs, sc = (prep.query_scale if prep.query_scale is not None else (0.0, 0.0))
-            mode = _RET_MODES[retention[0]]
+            mode = _ret_mode(retention)
             param = int(retention[1]) if len(retention) > 1 else 0
             self._call("jle_attention_decode_fused", _p(qkv), _p(kv_cache), _p(out), _p(ws_ml), _p(ws_o),
                        _p(self._tickets), _p(positions), _p(token_segment), _p(block_table), block_table.shape[1],
@@ -574,7 +582,7 @@ class HipOps:
         self._chk(block_table, torch.int32, None, "block table")
         self._chk(positions, torch.int32, (n,), "positions")
         self._chk(token_segment, torch.int32, (n,), "token segments")
-        mode = _RET_MODES[retention[0]]
+        mode = _ret_mode(retention)
         param = int(retention[1]) if len(retention) > 1 else 0
         out = torch.empty(n, hq * dh, dtype=q.dtype, device=q.device)
         if (q.dtype == torch.bfloat16 and hq // hk <= 32

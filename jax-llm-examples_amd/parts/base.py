@@ -1,8 +1,9 @@
 """Interfaces of the parts a layer is put together from, and their registries.
 
-Four kinds of part exist: *mixers* (what moves information between positions:
-attention here), *feed-forwards* (dense or routed experts), *norms* and
-*position encodings*.  Each is a class registered under a ``kind`` name and
+A layer is put together from four kinds of part: *mixers* (what moves information
+between positions: attention here), *feed-forwards* (dense or routed experts), *norms* and
+*position encodings*; a model has an *embedding* before its layers and an *output head*
+behind them.  Each is a class registered under a ``kind`` name and
 built from a :class:`~..config.specs.PartSpec`; none knows which model it is
 in.  A part declares its parameters (:class:`ParamSpec`), a mixer declares
 what it needs from the cache manager (:class:`CacheNeed`: pages of keys and
@@ -82,8 +83,8 @@ class CacheNeed:
     ``paged``: further per-token tensors in pages (see below).
     ``retention``: which earlier tokens a query at position ``p`` may still read:
     ``("all",)``; ``("chunk", C)``: those with ``pos >= (p // C) * C``;
-    ``("window", W)``: those with ``pos > p - W``.  Pages that hold only
-    tokens no later query can read are given back.
+    ``("window", W)``: those with ``pos > p - W``; or any rule registered with
+    :func:`register_retention`.  Pages that hold only tokens no later query can read are given back.
     ``state_shape``/``state_dtype``: fixed-size state per request (``None`` if the mixer has none).
     """
 
@@ -100,17 +101,57 @@ class CacheNeed:
     paged: tuple = ()
 
 
+@dataclasses.dataclass(frozen=True)
+class RetentionKind:
+    """What the cache manager has to know of a retention rule ``(kind, *parameters)``.
+
+    ``first_needed(rule, next_pos)``: the smallest position, beyond the kept prefix, that a query at
+    ``next_pos`` or later can still read.  ``held_at_most(rule, max_step_tokens)``: the most tokens of one
+    request that are held at any time (what the rule keeps plus one step's portion, whose pages are
+    given back only after the step), or ``None`` if only the sequence's length bounds it.
+    ``kept_prefix(rule)``: positions ``[0, kept_prefix)`` stay readable for ever."""
+
+    first_needed: Callable[[tuple, int], int]
+    held_at_most: Callable[[tuple, int], Optional[int]]
+    kept_prefix: Callable[[tuple], int] = lambda rule: 0
+
+
+_RETENTIONS: dict[str, RetentionKind] = {}
+
+
+def register_retention(kind: str, first_needed, held_at_most, kept_prefix=None) -> None:
+    """A further retention rule for mixers that read their pages themselves (the attention kernels here read
+    keys under ``all``, ``chunk`` and ``window``): the cache manager gives pages back by it and sizes pools by it."""
+    _RETENTIONS[kind] = RetentionKind(first_needed, held_at_most, kept_prefix or (lambda rule: 0))
+
+
+def retention_kind(retention: tuple) -> RetentionKind:
+    try:
+        return _RETENTIONS[retention[0]]
+    except KeyError:
+        raise ValueError(f"unknown retention rule {retention!r}; registered: {', '.join(sorted(_RETENTIONS))}") from None
+
+
+register_retention("all", lambda rule, next_pos: 0, lambda rule, step: None)
+register_retention("chunk", lambda rule, next_pos: (next_pos // int(rule[1])) * int(rule[1]),
+                   lambda rule, step: int(rule[1]) + step)
+register_retention("window", lambda rule, next_pos: max(0, next_pos - int(rule[1]) + 1),
+                   lambda rule, step: int(rule[1]) + step)
+
+
 def first_needed_position(retention: tuple, next_pos: int) -> int:
-    """Smallest position that a query at ``next_pos`` or later can still read."""
-    kind = retention[0]
-    if kind == "all":
-        return 0
-    if kind == "chunk":
-        c = int(retention[1])
-        return (next_pos // c) * c
-    if kind == "window":
-        return max(0, next_pos - int(retention[1]) + 1)
-    raise ValueError(f"unknown retention rule {retention!r}")
+    """Smallest position (beyond the rule's kept prefix) that a query at ``next_pos`` or later can still read."""
+    return retention_kind(retention).first_needed(retention, next_pos)
+
+
+def kept_prefix(retention: tuple) -> int:
+    return retention_kind(retention).kept_prefix(retention)
+
+
+def readable(retention: tuple, query_pos: int, key_pos: int) -> bool:
+    """The rule itself: may the query at ``query_pos`` read the key at ``key_pos``?"""
+    return key_pos <= query_pos and (key_pos < kept_prefix(retention)
+                                     or key_pos >= first_needed_position(retention, query_pos))
 
 
 # --------------------------------------------------------------------------- interfaces
@@ -158,6 +199,30 @@ class Norm(Part):
 
     def forward(self, residual: Any, ctx: Any, want32: bool = False):  # pragma: no cover
         raise NotImplementedError
+
+
+class Embedding(Part):
+    """``forward(token_ids, ctx)``: int32 ``[N]`` token ids to the first residual, float32 ``[N, hidden]``."""
+
+    def forward(self, token_ids: torch.Tensor, ctx: Any) -> torch.Tensor:  # pragma: no cover
+        raise NotImplementedError
+
+    def step_bytes(self, num_tokens: int) -> int:
+        """Bytes a step of ``num_tokens`` tokens reads of this part (a table: a row per token)."""
+        return sum(num_tokens * t.shape[-1] * t.element_size() for t in self.params.values() if t.dim() == 2)
+
+
+class OutputHead(Part):
+    """``forward(h, ctx, embedding)``: the normed rows ``[M, hidden]`` whose logits are wanted, in the run
+    dtype, to float32 logits ``[M, vocab]``.  ``embedding`` is the model's embedding part (a tied head takes
+    its matrix from there)."""
+
+    def forward(self, h: torch.Tensor, ctx: Any, embedding: Any) -> torch.Tensor:  # pragma: no cover
+        raise NotImplementedError
+
+    def step_bytes(self, embedding: Any) -> int:
+        """Bytes a step reads of the head's parameters (a tied head: of the embedding's)."""
+        return self.step_weight_bytes()
 
 
 @dataclasses.dataclass
@@ -214,6 +279,8 @@ _MIXERS: dict[str, Callable[..., Mixer]] = {}
 _FEED_FORWARDS: dict[str, Callable[..., FeedForward]] = {}
 _NORMS: dict[str, Callable[..., Norm]] = {}
 _POSITIONS: dict[str, Callable[..., PositionEncoding]] = {}
+_EMBEDDINGS: dict[str, Callable[..., Embedding]] = {}
+_HEADS: dict[str, Callable[..., OutputHead]] = {}
 
 
 def _register(table: dict, what: str):
@@ -238,3 +305,5 @@ register_mixer, build_mixer = _register(_MIXERS, "mixer")
 register_feed_forward, build_feed_forward = _register(_FEED_FORWARDS, "feed-forward")
 register_norm, build_norm = _register(_NORMS, "norm")
 register_position, build_position = _register(_POSITIONS, "position encoding")
+register_embedding, build_embedding = _register(_EMBEDDINGS, "embedding")
+register_head, build_head = _register(_HEADS, "output head")

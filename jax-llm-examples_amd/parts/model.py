@@ -1,6 +1,6 @@
 """The generic decoder: embedding, the layers of a plan run in the plan's order,
-final norm and output head (``llama4/llama4_jax/model.py:1186-1210``).  It is
-built from a :class:`~..config.specs.ModelPlan` alone."""
+final norm and output head (``llama4/llama4_jax/model.py:1186-1210``), each a part built from
+its :class:`~..config.specs.PartSpec`.  It is built from a :class:`~..config.specs.ModelPlan` alone."""
 from __future__ import annotations
 
 import torch
@@ -8,30 +8,10 @@ import torch
 from ..cache.manager import CacheView
 from ..config.specs import ModelPlan
 from .residual import Residual
-from .base import CacheNeed, ParamSpec, Part, build_norm
+from ..config.specs import part
+from . import embedding as _ends  # noqa: F401  (registers the built-in embedding and head)
+from .base import CacheNeed, ParamSpec, Part, build_embedding, build_head, build_norm
 from .block import build_block
-
-
-class _Table(Part):
-    def __init__(self, rows: int, cols: int) -> None:
-        super().__init__()
-        self.shape = (rows, cols)
-
-    def param_specs(self):
-        return {"weight": ParamSpec(self.shape)}
-
-
-class _Head(_Table):
-    """The output head: its matrix takes the product kernels' streaming layout where it can."""
-
-    tiled = False
-
-    def finalize(self) -> None:
-        from ..ops.layout import can_tile, tile_
-
-        if not self.tiled and can_tile(self.params["weight"]):
-            tile_(self.params["weight"])
-            self.tiled = True
 
 
 class DecoderModel:
@@ -39,10 +19,13 @@ class DecoderModel:
         self.plan = plan
         self.dtype = dtype
         self.device = torch.device(device)
-        self.embed = _Table(plan.vocab_size, plan.hidden_size)
+        # (a plan that does not describe its two ends gets a plain table and a plain linear head)
+        self.embed = build_embedding(plan.embedding or part("token_embedding", vocab_size=plan.vocab_size,
+                                                            hidden_size=plan.hidden_size))
         self.blocks = [build_block(spec) for spec in plan.layers]
         self.final_norm = build_norm(plan.final_norm)
-        self.lm_head = None if plan.tie_word_embeddings else _Head(plan.vocab_size, plan.hidden_size)
+        self.lm_head = build_head(plan.head or part("linear_head", vocab_size=plan.vocab_size,
+                                                    hidden_size=plan.hidden_size, tied=plan.tie_word_embeddings))
         self._allocated = False
 
     # ------------------------------------------------------------------ parameters
@@ -52,8 +35,7 @@ class DecoderModel:
             for name, p in b.parts().items():
                 out[f"layers.{i}.{name}"] = p
         out["final_norm"] = self.final_norm
-        if self.lm_head is not None:
-            out["lm_head"] = self.lm_head
+        out["lm_head"] = self.lm_head
         return out
 
     def param_specs(self) -> dict[str, ParamSpec]:
@@ -97,7 +79,7 @@ class DecoderModel:
         """Runs the step's tokens through every run of the order; returns float32
         logits ``[len(ctx.logits_indices), vocab]``."""
         ops = ctx.ops
-        residual = Residual(ops.embed(ctx.token_ids, self.embed.params["weight"]))
+        residual = Residual(self.embed.forward(ctx.token_ids, ctx))
         for e in self.plan.order:
             gi = cache.group_of.get(e.cache)
             view = CacheView(cache_id=e.cache, writes=e.writes_cache, group=gi, state=cache.state.get(e.cache))
@@ -114,5 +96,4 @@ class DecoderModel:
             return torch.empty(0, self.plan.vocab_size, dtype=torch.float32, device=ctx.device)
         picked = residual.rows(ctx, ctx.logits_indices)
         h, _ = self.final_norm.forward(picked, ctx)
-        head = self.embed if self.lm_head is None else self.lm_head
-        return ops.lm_head(h, head.params["weight"], tiled=getattr(head, "tiled", False))
+        return self.lm_head.forward(h, ctx, self.embed)

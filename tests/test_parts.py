@@ -524,6 +524,146 @@ def test_half_split_partial_rotary_with_weighted_norm_and_pages_of_other_shapes(
     assert torch.allclose(torch.cat(outs), direct, rtol=1e-4, atol=2e-5)
 
 
+# ---------------------------------------- a retention rule of its own: the first tokens for ever, plus a window
+def _register_sink_window():
+    from jax_llm_examples_amd.parts import register_retention
+    register_retention("toy_sink_window",
+                       first_needed=lambda rule, next_pos: max(0, next_pos - int(rule[2]) + 1),
+                       held_at_most=lambda rule, step: int(rule[1]) + int(rule[2]) + step,
+                       kept_prefix=lambda rule: int(rule[1]))
+
+
+_register_sink_window()
+
+
+@register_mixer("toy_sink_mean")
+class ToySinkMean(Mixer):
+    """The mean of a per-token value over the first ``sink`` positions and the last ``window``: a rule for which
+    keys stay readable that the framework does not know, registered above.  Plain PyTorch over the block table."""
+
+    def __init__(self, spec):
+        super().__init__()
+        self.hidden, self.sink, self.window = int(spec.hidden_size), int(spec.sink), int(spec.window)
+
+    def param_specs(self):
+        return {"w": ParamSpec((self.hidden, self.hidden))}
+
+    def cache_need(self):
+        return CacheNeed(paged=(("value", (self.hidden,)),), retention=("toy_sink_window", self.sink, self.window))
+
+    def forward(self, h, ctx, cache):
+        from jax_llm_examples_amd.parts.base import readable
+        ps, rule = ctx.page_size, self.cache_need().retention
+        flat = cache.pages["value"].view(-1, self.hidden)
+        flat[cache.slot_mapping.long()] = h.to(flat.dtype)
+        out = torch.empty_like(h)
+        for i, (p, sg) in enumerate(zip(ctx.positions.tolist(), ctx.token_segment.tolist())):
+            keys = torch.tensor([k for k in range(p + 1) if readable(rule, p, k)], device=h.device)
+            pages = cache.block_table[sg][(keys // ps).long()].long()
+            assert bool((pages >= 0).all()), "a readable key's page was given back"
+            out[i] = (self.params["w"].float() @ flat[pages * ps + keys % ps].float().mean(0)).to(h.dtype)
+        return out
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_a_retention_rule_defined_here_keeps_a_prefix_and_a_window(device):
+    """The cache manager gives back exactly the pages between the kept prefix and the window, sizes the pool by
+    the rule, and the mixer's result does not depend on the cut (pool poisoned: a page given back too early
+    would show)."""
+    from jax_llm_examples_amd.cache import pool_sizes
+    D = 24
+    norm = part("rmsnorm", eps=1e-5, weighted=True, size=D)
+    layer = LayerSpec(mixer=part("toy_sink_mean", hidden_size=D, sink=6, window=9),
+                      feed_forward=part("dense_swiglu", hidden_size=D, intermediate_size=16),
+                      mixer_norm=norm, feed_forward_norm=norm)
+    plan = ModelPlan(vocab_size=53, hidden_size=D, layers=(layer,), order=(OrderEntry(0, 0),), final_norm=norm)
+    model = DecoderModel(plan, torch.float32, device)
+    model.allocate()
+    init_random_(model, seed=3, std=0.3)
+    needs = model.cache_needs()
+    sizes = pool_sizes(needs, page_size=4, itemsize=4, max_requests=3, max_step_tokens=20, cache_tokens=10_000)
+    assert sizes == {0: 3 * (-(-(6 + 9 + 20) // 4) + 1)}  # what the rule can hold, not what was asked for
+    reqs = traces.random_requests(53, [60, 33, 47], seed=4)
+    results = {}
+    for mode in ("whole", "tail", "portions", "mixed"):
+        cache = CacheManager(needs, page_size=4, num_pages=60, max_requests=3, dtype=torch.float32, device=device,
+                             poison=True)
+        runner = ModelRunner(model, cache, _ops(device))
+        results[mode] = traces.run_trace(runner, getattr(traces, mode)(reqs))
+        cache.check()
+    for rid in reqs:
+        assert torch.isfinite(results["whole"][rid]).all()
+        for mode in ("tail", "portions", "mixed"):
+            assert torch.allclose(results[mode][rid], results["whole"][rid], rtol=1e-4, atol=1e-5), (mode, rid)
+    # which pages a request holds after 41 tokens: those of positions 0..5 (pages 0, 1) and 33..40 (pages 8..10)
+    cache = CacheManager(needs, page_size=4, num_pages=60, max_requests=1, dtype=torch.float32, device="cpu")
+    cache.add_request("a")
+    for n in (17, 1, 1, 22):
+        cache.reserve("a", n)
+        cache.commit("a")
+    held = [j for j, pg in enumerate(cache.table("a", 0)) if pg >= 0]
+    assert held == [0, 1, 8, 9, 10]
+    with pytest.raises(ValueError, match="unknown retention rule"):
+        CacheManager({0: CacheNeed(kv=(1, 8), retention=("nothing_like_it", 3))}, page_size=4, num_pages=4,
+                     max_requests=1, dtype=torch.float32, device="cpu")
+
+
+# ---------------------------------------------------- the model's two ends are parts too
+@pytest.mark.parametrize("device", DEVICES)
+def test_embedding_and_head_are_parts_with_options_and_may_be_replaced(device):
+    """A scaled embedding, a tied head with a bias and a soft cap (said in the plan), and a head of another kind
+    registered here: no framework file is touched."""
+    from jax_llm_examples_amd.parts import OutputHead, register_head
+
+    @register_head("toy_sign_head")
+    class ToySignHead(OutputHead):
+        def __init__(self, spec):
+            super().__init__()
+            self.vocab_size = int(spec.vocab_size)
+
+        def forward(self, h, ctx, embedding):
+            logits = h.float() @ embedding.params["weight"].float().t()
+            return torch.sign(logits) * logits.abs().sqrt()
+
+    D, V = 16, 37
+    norm = part("rmsnorm", eps=1e-5, weighted=True, size=D)
+    layer = LayerSpec(mixer=part("toy_decayed_sum", hidden_size=D, decay=0.5),
+                      feed_forward=part("dense_swiglu", hidden_size=D, intermediate_size=8),
+                      mixer_norm=norm, feed_forward_norm=norm)
+
+    def build(embedding, head):
+        plan = ModelPlan(vocab_size=V, hidden_size=D, layers=(layer,), order=(OrderEntry(0, 0),), final_norm=norm,
+                         embedding=embedding, head=head)
+        model = DecoderModel(plan, torch.float32, device)
+        model.allocate()
+        init_random_(model, seed=5, std=0.3)
+        return model
+
+    def logits(model, toks):
+        cache = CacheManager(model.cache_needs(), page_size=4, num_pages=4, max_requests=1, dtype=torch.float32,
+                             device=device)
+        runner = ModelRunner(model, cache, _ops(device))
+        return runner.step([StepEntry("r", toks, list(range(len(toks))))]).float().cpu()
+
+    toks = [3, 30, 7, 7, 12]
+    plain = build(None, None)
+    assert set(plain.named_parameters()) >= {"embed.weight", "lm_head.weight"}
+    base = logits(plain, toks)
+    tied = build(part("token_embedding", vocab_size=V, hidden_size=D, multiplier=2.0),
+                 part("linear_head", vocab_size=V, hidden_size=D, tied=True, bias=True, softcap=3.0))
+    names = set(tied.named_parameters())
+    assert "lm_head.weight" not in names and "lm_head.bias" in names
+    got = logits(tied, toks)
+    assert got.abs().max() <= 3.0 and not torch.allclose(got, base)
+    # the same by hand from the model's own pieces: embedding times 2 ... head over the embedding's table
+    x = tied.embed.params["weight"][torch.tensor(toks)].float().cpu() * 2.0
+    assert torch.allclose(tied.embed.forward(torch.tensor(toks, dtype=torch.int32, device=device),
+                                             type("C", (), {"ops": _ops(device)})()).cpu(), x)
+    signed = build(None, part("toy_sign_head", vocab_size=V))
+    assert isinstance(signed.lm_head, ToySignHead) and "lm_head.weight" not in signed.named_parameters()
+    assert torch.isfinite(logits(signed, toks)).all()
+
+
 def test_order_is_checked():
     norm = part("rmsnorm", eps=1e-5, weighted=True, size=8)
     layer = LayerSpec(part("toy_decayed_sum", hidden_size=8, decay=0.5),
