@@ -250,3 +250,17 @@ JLE_API int jle_paged_attention_generic(const void* q, const void* kv, void* out
   JLE_LAUNCH_CHECK();
   return 0;
 }
+
+// The merge alone, for kernels that leave their key ranges' results in the same layout (attention_f32.hip).
+JLE_API int jle_attention_merge(const float* ws_ml, const float* ws_o, void* out, int is_bf16, int NH, int dh,
+                                int splits, hipStream_t s) {
+  if (NH <= 0) return 0;
+  if (splits < 1 || dh <= 0 || dh > 256 || ws_ml == nullptr || ws_o == nullptr) return JLE_BAD_ARG;
+  dim3 gm((unsigned)(((long long)NH + 3) / 4)), b(256);
+  if (is_bf16)
+    hipLaunchKernelGGL(paged_attention_generic_merge_kernel<bf16_t>, gm, b, 0, s, ws_ml, ws_o, (bf16_t*)out, NH, dh, splits);
+  else
+    hipLaunchKernelGGL(paged_attention_generic_merge_kernel<float>, gm, b, 0, s, ws_ml, ws_o, (float*)out, NH, dh, splits);
+  JLE_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,146 @@
+// Grouped weight-streaming matrix product in true float32 on the matrix cores (v_mfma_f32_16x16x4_f32: float32
+// operands, float32 products and sums; no reduced-precision mode anywhere): what the float32 run of the model
+// uses for its routed experts in steps of few tokens.
+//
+//   Y[t, n] = scale[t] * sum_k X[arow(t), k] * W[g(t)][n, k]                         (plain)
+//   Y[t, f] = silu(s * gate) * (s * up), gate / up = rows f and F + f of W[g(t)]      (SWIGLU)
+//
+// Rows t are sorted by group: offsets[g] .. offsets[g + 1] use W[g] (offsets == nullptr: one group).  W is
+// row-major [G][Nout][K].
+//
+// Few rows (decode; a group's rows in tiles of 16): the cost is reading W once.  The weights are the A operand,
+// the tokens' rows the B operand.  The wavefronts of a block split K (every 8th chunk of 32 k each) and add their
+// sums in shared memory in a fixed order.  (With many rows per group the general float32 kernel of
+// gemm_generic.hip is the faster one: a 128 x 128 x 32 tiled kernel on these instructions reached 44 to 63
+// TFLOP/s at 128 to 512 rows per expert where that one reaches 58 to 70, and was taken out again.)
+//
+// Order of the sums: an element's sum over k is formed per wavefront over its chunks in ascending order, within
+// a chunk in the order of the instruction's 4 k-lanes and the lane's 8 elements; the wavefronts' sums are added
+// in wavefront order.  It depends on K only, not on the number of rows or groups.
+#include "common.h"
+
+using namespace jle;
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+namespace {
+
+__device__ __forceinline__ float silu_mul(float gate, float up) { return gate / (1.0f + expf(-gate)) * up; }
+
+// 16 bytes that the caches need not keep (weights are read once)
+__device__ __forceinline__ float4 load_once(const float* p) {
+  const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+  return float4{v[0], v[1], v[2], v[3]};
+}
+
+// ------------------------------------------------------------------------------------------------ few rows
+constexpr int kSkinnyWaves = 8;
+constexpr int kSkinnyChunks = 4;  // chunks of 32 k on their way per wavefront
+
+// A lane reads 8 consecutive floats of its weight row (two 16-byte loads; the 4 lanes of a row read one whole
+// 128-byte line between them, a wavefront 16 rows x 32 k), which feed 8 instructions; the lane of the B operand
+// reads the same 8 k of its token's row.  (Dealing the lanes so that every single load instruction covers whole
+// lines - 8 rows x 128 bytes, the even and the odd 16-byte pieces of a row multiplied in instructions of their
+// own - was measured slower: 805 + 442 us a layer against 622 + 286 for Scout's experts at batch 8.)
+template <bool SWIGLU>
+__global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
+    const float* __restrict__ X, const float* __restrict__ W, float* __restrict__ Y, const int* __restrict__ offsets,
+    const int* __restrict__ a_rows, const float* __restrict__ scale, int M, int Nout, int K) {
+  constexpr int RT = SWIGLU ? 2 : 1;
+  __shared__ float red[kSkinnyWaves][RT * 4][64];
+  const int e = blockIdx.z;
+  int row_lo = 0, row_hi = M;
+  if (offsets != nullptr) {
+    row_lo = offsets[e];
+    row_hi = offsets[e + 1];
+  }
+  const int tok0 = row_lo + blockIdx.y * 16;
+  if (tok0 >= row_hi) return;  // the whole block
+  const int lane = threadIdx.x & 63, wave = wave_index();
+  const int r = lane & 15, g = lane >> 4;
+  const float* We = W + (size_t)e * Nout * K;
+  const int half = Nout >> 1;
+  const int base = blockIdx.x * 16;  // first output column of the block
+  const int cols = SWIGLU ? half : Nout;
+  const int wrow0 = min(base + r, cols - 1);
+  const float* w0 = We + (size_t)wrow0 * K + 8 * g;
+  const float* w1 = We + (size_t)(wrow0 + half) * K + 8 * g;  // (SWIGLU: the up row of the gate row)
+  const int t = tok0 + r;
+  const bool xv = t < row_hi;
+  const float* xb = X + (size_t)(xv ? (a_rows != nullptr ? a_rows[t] : t) : 0) * K + 8 * g;
+  f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  const int nchunks = (K + 31) >> 5;
+  const float4 zero = {0.f, 0.f, 0.f, 0.f};
+  for (int c0 = wave; c0 < nchunks; c0 += kSkinnyWaves * kSkinnyChunks) {
+    float4 a0[kSkinnyChunks][2], a1[kSkinnyChunks][2], b[kSkinnyChunks][2];
+#pragma unroll
+    for (int u = 0; u < kSkinnyChunks; ++u) {
+      const int c = c0 + kSkinnyWaves * u;
+      const int k = c * 32 + 8 * g;
+      // K is a multiple of 4: the lane's 8 floats are two pieces of 4, each inside the row or not at all
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const bool ok = c < nchunks && k + 4 * h < K;
+        a0[u][h] = ok ? load_once(w0 + (size_t)c * 32 + 4 * h) : zero;
+        if (SWIGLU) a1[u][h] = ok ? load_once(w1 + (size_t)c * 32 + 4 * h) : zero;
+        b[u][h] = (ok && xv) ? *reinterpret_cast<const float4*>(xb + (size_t)c * 32 + 4 * h) : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kSkinnyChunks; ++u) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const float av[4] = {a0[u][h].x, a0[u][h].y, a0[u][h].z, a0[u][h].w};
+        const float uv[4] = {a1[u][h].x, a1[u][h].y, a1[u][h].z, a1[u][h].w};
+        const float bv[4] = {b[u][h].x, b[u][h].y, b[u][h].z, b[u][h].w};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s], bv[s], acc0, 0, 0, 0);
+          if (SWIGLU) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(uv[s], bv[s], acc1, 0, 0, 0);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    red[wave][i][lane] = acc0[i];
+    if (SWIGLU) red[wave][4 + i][lane] = acc1[i];
+  }
+  __syncthreads();
+  // wavefront w < 4 finishes element i = w: D[row 4 * g + i of the tile][token r]
+  if (wave >= 4) return;
+  const int i = wave;
+  float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+  for (int w = 0; w < kSkinnyWaves; ++w) {
+    v0 += red[w][i][lane];
+    if (SWIGLU) v1 += red[w][4 + i][lane];
+  }
+  if (!xv) return;
+  const float sc = scale != nullptr ? scale[t] : 1.f;
+  const int col = base + 4 * g + i;
+  if (col >= cols) return;
+  if (SWIGLU) Y[(size_t)t * half + col] = silu_mul(v0 * sc, v1 * sc);
+  else Y[(size_t)t * Nout + col] = v0 * sc;
+}
+
+}  // namespace
+
+// X [*, K], W [G, Nout, K], Y [M, Nout] (or [M, Nout / 2] with swiglu), all float32; K a multiple of 4 and every
+// row 16-byte aligned.  max_rows: the most rows any group can have (M if unknown).
+JLE_API int jle_gemm_f32_skinny(const float* X, const float* W, float* Y, const int* offsets, const int* a_rows,
+                                const float* scale, int swiglu, int M, int Nout, int K, int G, int max_rows,
+                                hipStream_t s) {
+  if (M <= 0 || Nout <= 0) return 0;
+  if (K <= 0 || K % 4 || G < 1 || G > 65535 || (swiglu && Nout % 2)) return JLE_BAD_ARG;
+  if ((((uintptr_t)X | (uintptr_t)W | (uintptr_t)Y) & 15) != 0) return JLE_BAD_ARG;
+  if (max_rows <= 0 || max_rows > M) max_rows = M;
+  const int cols = swiglu ? Nout / 2 : Nout;
+  const int ytiles = (max_rows + 15) / 16;
+  if (ytiles > 65535) return JLE_BAD_ARG;
+  dim3 g((cols + 15) / 16, ytiles, offsets != nullptr ? G : 1), b(kSkinnyWaves * 64);
+  if (swiglu) hipLaunchKernelGGL(gemm_f32_skinny_kernel<true>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);
+  else hipLaunchKernelGGL(gemm_f32_skinny_kernel<false>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);
+  JLE_LAUNCH_CHECK();
+  return 0;
+}

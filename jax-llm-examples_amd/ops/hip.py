@@ -36,12 +36,16 @@ _SIGNATURES = {
                        _vp],
     "jle_paged_attention_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _i, _i, _vp,
                                     _vp, _vp],
+    "jle_attention_f32_tiles": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
+    "jle_attention_f32_heads": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp],
+    "jle_attention_merge": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_moe_route": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_norm_route": [_vp, _i, _vp, _vp, _vp, _i, _vp, _i, _vp, _f, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                        _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_moe_route_align": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_f32_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
     "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
@@ -273,6 +277,29 @@ class HipOps:
         out = torch.empty(m, nout, dtype=torch.float32 if out_f32 else a.dtype, device=a.device)
         self._call("jle_gemm_generic", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), self._is_bf16(a),
                    1 if (out_f32 or a.dtype == torch.float32) else 0, m, nout, k, g)
+        return out
+
+    F32_SKINNY_ROWS = 128  # float32 grouped products: up to so many rows the weight-streaming kernel on the float32
+    # matrix instructions; beyond, the general kernel (measured faster there than a tiled kernel on those instructions)
+
+    def gemm_f32_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, rows=None):
+        """The float32 grouped product for few rows on the float32 matrix instructions (see ``gemm_f32.hip``):
+        float32 operands, products and sums.  With ``swiglu`` the result is ``silu(gate) * up`` of the two halves
+        of ``b``'s rows."""
+        if b.dim() == 2:
+            b = b.unsqueeze(0)
+        g, nout, k = b.shape
+        m = rows if rows is not None else (a_rows.numel() if a_rows is not None else a.shape[0])
+        self._chk(a, torch.float32, None, "A")
+        self._chk(b, torch.float32, None, "B")
+        if a.shape[1] != k:
+            raise KernelError(f"inner sizes differ: A {tuple(a.shape)}, B {tuple(b.shape)}")
+        if k % 4 or a.data_ptr() % 16 or b.data_ptr() % 16:
+            raise KernelError(f"the float32 matrix-core product needs an inner size that is a multiple of 4 and "
+                              f"16-byte aligned rows, got K = {k}")
+        out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32, device=a.device)
+        self._call("jle_gemm_f32_skinny", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu), m,
+                   nout, k, g, m)
         return out
 
     SKINNY_MAX_ROWS = 64  # up to here a product is a stream of the weights: the MFMA weight-streaming kernel
@@ -574,6 +601,25 @@ class HipOps:
                 "dec": flat[:nd] if dec else None, "tiles": flat[nd: nd + nt] if tiles else None,
                 "groups": flat[nd + nt:] if groups else None, "num_groups": len(groups) // 4}
 
+    @staticmethod
+    def _segments(meta, token_segment, positions):
+        """The step's segments (lengths, first positions): from the step's context or, in a direct call (tests),
+        recovered from the device arrays."""
+        if meta is not None and meta.seg_starts is not None:
+            return meta.seg_lens, meta.seg_starts
+        seg = token_segment.cpu().tolist()
+        pos = positions.cpu().tolist()
+        seg_lens, seg_starts = [], []
+        for i, sgm in enumerate(seg):
+            if i == 0 or sgm != seg[i - 1]:
+                seg_lens.append(0)
+                seg_starts.append(pos[i])
+            seg_lens[-1] += 1
+        return seg_lens, seg_starts
+
+    F32_TILE = 16  # tokens per work item of the float32 matrix-instruction attention
+    F32_DECODE_ITEMS = 2048  # ... in a step of single tokens: about so many (token, kv head, key range) items
+
     def paged_attention(self, q, kv_cache, block_table, positions, token_segment, retention, scale: float, meta=None):
         n, hq, dh = q.shape
         hk, ps = kv_cache.shape[2], kv_cache.shape[3]
@@ -590,17 +636,7 @@ class HipOps:
             key = f"attn_plan_{hq // hk}"
             plan = meta.meta.get(key) if meta is not None else None
             if plan is None:
-                if meta is not None:
-                    seg_lens, seg_starts = meta.seg_lens, meta.seg_starts
-                else:  # a direct call (tests): recover the segments from the device arrays
-                    seg = token_segment.cpu().tolist()
-                    pos = positions.cpu().tolist()
-                    seg_lens, seg_starts = [], []
-                    for i, sgm in enumerate(seg):
-                        if i == 0 or sgm != seg[i - 1]:
-                            seg_lens.append(0)
-                            seg_starts.append(pos[i])
-                        seg_lens[-1] += 1
+                seg_lens, seg_starts = self._segments(meta, token_segment, positions)
                 plan = self.attention_plan(seg_lens, seg_starts, retention, q.device, hk, hq // hk,
                                            decode_bucket=meta.decode_bucket if meta is not None else None)
                 if meta is not None:
@@ -623,6 +659,47 @@ class HipOps:
             raise KernelError(f"attention kernels: head size {dh} is not supported (a multiple of 8, at most 256)")
         if hq % hk:
             raise KernelError(f"attention kernels: {hq} query heads are no multiple of {hk} kv heads")
+        if (q.dtype == torch.float32 and dh % 16 == 0 and ps % 16 == 0 and n * hq >= self.GENERIC_SPLIT_BELOW
+                and (meta is None or meta.decode_bucket is None)):
+            # many tokens in float32: tiles of 16 tokens on the float32 matrix instructions
+            tiles = meta.meta.get("f32_tiles") if meta is not None else None
+            if tiles is None:
+                seg_lens, _ = self._segments(meta, token_segment, positions)
+                flat, o = [], 0
+                for ln in seg_lens:
+                    for t in range(0, ln, self.F32_TILE):
+                        flat += [o + t, min(self.F32_TILE, ln - t)]
+                    o += ln
+                tiles = torch.tensor(flat, dtype=torch.int32).to(q.device)
+                if meta is not None:
+                    meta.meta["f32_tiles"] = tiles
+            self._call("jle_attention_f32_tiles", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
+                       _p(block_table), block_table.shape[1], _p(tiles), tiles.numel() // 2, mode, param, float(scale),
+                       hq, hk, dh, ps)
+            return out
+        if (q.dtype == torch.float32 and dh % 16 == 0 and ps % 16 == 0 and hq // hk <= 16
+                and ((meta is not None and meta.decode_bucket is not None)
+                     or all(ln == 1 for ln in self._segments(meta, token_segment, positions)[0]))):
+            # a step of single tokens in float32: the query heads of a kv head share a wavefront (its keys and
+            # values are read once for all of them), the keys are shared between wavefronts and merged
+            if meta is not None and meta.decode_bucket is not None:
+                longest = meta.decode_bucket
+            else:
+                longest = int(positions.max()) + 1
+            steps = -(-longest // 64)
+            want = max(1, min(steps, -(-self.F32_DECODE_ITEMS // (n * hk))))
+            per = -(-steps // want) * 64
+            splits = -(-longest // per)
+            ws_ml = ws_o = None
+            if splits > 1:
+                ws_ml = torch.empty(n * hq * splits * 2, dtype=torch.float32, device=q.device)
+                ws_o = torch.empty(n * hq * splits * dh, dtype=torch.float32, device=q.device)
+            self._call("jle_attention_f32_heads", _p(q), _p(kv_cache), _p(out), _p(positions), _p(token_segment),
+                       _p(block_table), block_table.shape[1], n, mode, param, float(scale), hq, hk, dh, ps, splits,
+                       per, _p(ws_ml), _p(ws_o))
+            if splits > 1:
+                self._call("jle_attention_merge", _p(ws_ml), _p(ws_o), _p(out), 0, n * hq, dh, splits)
+            return out
         # few tokens with many keys (decode): each query's keys are shared between several wavefronts
         splits, tiles_per_split, ws_ml, ws_o = 1, 0, None, None
         waves = n * hq
@@ -781,6 +858,12 @@ class HipOps:
             routed = self.gemm_grouped(act, w_down, offsets=offsets, tiled=tiled)
         elif tiled:
             raise KernelError("weights in the streaming layout need the MFMA product kernels")
+        elif h.dtype == torch.float32 and d % 4 == 0 and (f2 // 2) % 4 == 0 and m <= self.F32_SKINNY_ROWS:
+            # few rows in true float32: the weights streamed once through the float32 matrix instructions, the
+            # activation fused into the first product
+            act = self.gemm_f32_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate,
+                                       swiglu=True)
+            routed = self.gemm_f32_skinny(act, w_down, offsets=offsets)
         else:
             gu = self.gemm(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate)
             act = self.silu_mul(gu)

@@ -211,6 +211,52 @@ def test_paged_attention(ops, ref, dt, hq, hk, dh, ps, retention):
     _assert_close_to_scale(got, want, dt)
 
 
+@pytest.mark.parametrize("hq,hk,dh,ps", [(4, 2, 16, 16), (5, 1, 48, 16), (8, 8, 64, 16), (10, 2, 128, 16), (2, 1, 256, 32),
+                                         (3, 1, 80, 16), (20, 1, 96, 48), (9, 3, 128, 48), (5, 5, 64, 64)])
+@pytest.mark.parametrize("retention", [("all",), ("chunk", 24), ("chunk", 100), ("window", 37)])
+def test_float32_attention_of_portions_on_the_float32_matrix_instructions(ops, ref, monkeypatch, hq, hk, dh, ps, retention):
+    """Tiles of 16 tokens per wavefront (steps of many tokens in float32 take this kernel): portions that start
+    anywhere, single tokens between them, keys of earlier steps; and a token's result does not depend on which
+    tile it falls into."""
+    monkeypatch.setattr(type(ops), "GENERIC_SPLIT_BELOW", 0)
+    specs = [(0, 70), (130, 1), (45, 9), (63, 2), (200, 1), (600, 1), (255, 35)]
+    q, kv, bt, pos, seg = _attention_case(hq, hk, dh, ps, torch.float32, specs)
+    calls = []
+    inner = ops._call
+    monkeypatch.setattr(ops, "_call", lambda name, *a: (calls.append(name), inner(name, *a))[1])
+    got = ops.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
+    assert calls == ["jle_attention_f32_tiles"]
+    want = ref.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
+    _assert_close_to_scale(got, want, torch.float32)
+    # the last 20 tokens of the last portion alone (other tiles, an odd start): the same bits
+    n = q.shape[0]
+    alone = ops.paged_attention(q[n - 20:].contiguous(), kv, bt, pos[n - 20:].contiguous(), seg[n - 20:].contiguous(),
+                                retention, dh ** -0.5)
+    assert torch.equal(alone, got[n - 20:])
+
+
+@pytest.mark.parametrize("hq,hk,dh,ps", [(4, 2, 16, 16), (5, 1, 48, 16), (40, 8, 128, 16), (16, 1, 64, 32), (3, 3, 256, 16)])
+@pytest.mark.parametrize("retention", [("all",), ("chunk", 100), ("window", 37)])
+def test_float32_attention_of_single_tokens_on_the_float32_matrix_instructions(ops, ref, monkeypatch, hq, hk, dh, ps, retention):
+    """A step of single tokens in float32: the query heads of a kv head share a wavefront, the keys are shared
+    between wavefronts (forced here to ranges of 64 keys, so that every token has several) and merged."""
+    monkeypatch.setattr(type(ops), "F32_DECODE_ITEMS", 1 << 20)
+    specs = [(130, 1), (0, 1), (63, 1), (200, 1), (600, 1), (15, 1), (99, 1)]
+    q, kv, bt, pos, seg = _attention_case(hq, hk, dh, ps, torch.float32, specs)
+    calls = []
+    inner = ops._call
+    monkeypatch.setattr(ops, "_call", lambda name, *a: (calls.append(name), inner(name, *a))[1])
+    got = ops.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
+    assert calls == ["jle_attention_f32_heads", "jle_attention_merge"]
+    want = ref.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
+    _assert_close_to_scale(got, want, torch.float32)
+    monkeypatch.setattr(type(ops), "F32_DECODE_ITEMS", 1)  # one range per token: no merge
+    calls.clear()
+    whole = ops.paged_attention(q, kv, bt, pos, seg, retention, dh ** -0.5)
+    assert calls == ["jle_attention_f32_heads"]
+    _assert_close_to_scale(whole, want, torch.float32)
+
+
 @pytest.mark.parametrize("hq,hk,ps", [(10, 2, 16), (40, 8, 16), (6, 3, 32), (9, 3, 48), (4, 2, 64)])
 @pytest.mark.parametrize("retention", [("all",), ("chunk", 192), ("chunk", 100), ("window", 150)])
 def test_paged_attention_of_long_portions_at_head_size_128(ops, ref, hq, hk, ps, retention):
@@ -635,6 +681,38 @@ def test_float32_products_are_true_float32_at_serving_sizes(ops, rows, k):
         assert float((out.double() - exact).abs().max()) <= 1e-6 * exact, name
         err = float(((fn(ar, br).double() - want).abs() / scale).max())
         assert err < 2e-6, f"{name}: {err:.3g} of the sum of the terms' sizes"
+
+
+@pytest.mark.parametrize("n,d,f,e,k", [(1, 64, 32, 4, 1), (8, 5120, 96, 16, 1), (64, 260, 36, 128, 2), (100, 128, 64, 5, 1),
+                                       (128, 512, 256, 16, 1), (50, 1028, 44, 3, 2), (129, 64, 16, 1, 1)])
+def test_float32_grouped_product_on_the_float32_matrix_instructions(ops, n, d, f, e, k):
+    """The weight-streaming float32 product (gemm_f32.hip) against float64: grouped, gathered, scaled, with and
+    without the fused activation; sizes that leave partial tiles, chunks and groups without rows."""
+    h = _rand(n, d, seed=1)
+    wgu, wd = _rand(e, 2 * f, d, scale=0.1, seed=2), _rand(e, d, f, scale=0.1, seed=3)
+    g = torch.Generator().manual_seed(n)
+    ids = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(n)]).to(torch.int32).to(DEV)
+    if e > 2:
+        ids[ids == 1] = 2  # a group without rows
+    gates = torch.rand(n, k, generator=g).to(DEV)
+    off, tok, gate, inv = ops.moe_align(ids, gates, e)
+    act = ops.gemm_f32_skinny(h, wgu, offsets=off, a_rows=tok, scale=gate, swiglu=True)
+    gu = ops.gemm_f32_skinny(h, wgu, offsets=off, a_rows=tok, scale=gate)
+    sorted_ids = ids.flatten()[torch.argsort(inv.long())].long()
+    x64 = h.double()[tok.long()] * gate.double()[:, None]
+    want_gu = torch.einsum("nk,nok->no", x64, wgu.double()[sorted_ids])
+    want_act = torch.nn.functional.silu(want_gu[:, :f]) * want_gu[:, f:]
+    assert float((gu.double() - want_gu).abs().max() / want_gu.abs().max()) <= 3e-6
+    assert float((act.double() - want_act).abs().max() / want_act.abs().max()) <= 3e-6
+    out = ops.gemm_f32_skinny(act, wd, offsets=off)
+    want = torch.einsum("nk,nok->no", act.double(), wd.double()[sorted_ids])
+    assert float((out.double() - want).abs().max() / want.abs().max()) <= 3e-6
+    # one group without offsets, and the result of a row does not depend on what else is in the launch
+    dense = ops.gemm_f32_skinny(h, wgu[0])
+    assert float((dense.double() - h.double() @ wgu[0].double().t()).abs().max() / dense.abs().max()) <= 3e-6
+    assert torch.equal(ops.gemm_f32_skinny(h[:1].contiguous(), wgu[0]), dense[:1])
+    with pytest.raises(Exception, match="multiple of 4"):
+        ops.gemm_f32_skinny(h[:, : d - 2].contiguous(), wgu[:, :, : d - 2].contiguous())
 
 
 def test_sampling(ops, ref):
