@@ -139,12 +139,20 @@ def main() -> int:
             one()
         torch.cuda.synchronize()
         sec = (time.perf_counter() - t1) / steps
-        watcher = StepWatcher()  # one more step, watched: which experts its tokens choose
-        one(tap=watcher)
-        distinct = {li: int(torch.unique(seen["routing"][0]).numel()) for li, b in enumerate(model.blocks)
-                    for seen in [watcher.seen.get(id(b.feed_forward))] if seen and "routing" in seen}
-        contexts = [cache.num_tokens(r) for r in ids]
-        nbytes = decode_step_bytes(model, cache, contexts, watcher)
+        # three more steps, watched: which experts their tokens choose (a watched step runs launch by launch);
+        # the step's bytes are the mean over them (the count of distinct experts wanders from step to step)
+        totals, weights_b, kv_b, counts = [], [], [], []
+        for _ in range(3):
+            watcher = StepWatcher()
+            one(tap=watcher)
+            counts += [int(torch.unique(seen["routing"][0]).numel()) for b in model.blocks
+                       for seen in [watcher.seen.get(id(b.feed_forward))] if seen and "routing" in seen]
+            nb = decode_step_bytes(model, cache, [cache.num_tokens(r) for r in ids], watcher)
+            totals.append(nb["total"])
+            weights_b.append(nb["weights"])
+            kv_b.append(nb["kv"])
+        nbytes = {"total": sum(totals) / 3, "weights": sum(weights_b) / 3, "kv": sum(kv_b) / 3}
+        distinct = {i: c for i, c in enumerate(counts)}
         for rid in ids:
             runner.finish(rid)
         print(f"[bench] decode batch {batch} at context {context}: {sec * 1e3:.2f} ms/step, {batch / sec:.1f} tok/s, "
