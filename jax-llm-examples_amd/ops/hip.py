@@ -308,6 +308,7 @@ class HipOps:
     SHARED_RIDES_ROWS = 16  # a shared expert's two products ride in the routed experts' launches as one more group
 
     SLICE_TICKETS = 1 << 14
+    CUT_SLOTS = 2  # a grouped launch has its row tiles cut along K only with so many group slots at most
     SLICE_ROWS = 16  # up to so many rows the row tiles of a launch may be cut along K (see _k_slices)
     SLOT_ROWS = 16  # a grouped product of so few rows is launched over as many group slots as it has rows
 
@@ -355,7 +356,9 @@ class HipOps:
         if balance and m <= self.SLICE_ROWS and variant <= 0:
             if offsets is not None and g > m and g <= 4096 and m <= self.SLOT_ROWS:
                 slots = m  # (no more groups have rows than there are rows)
-            if not swiglu and (offsets is None or slots):
+            # (several groups' tiles together fill their rounds well enough: measured at 2 to 8 tokens over 16
+            # experts and a shared one, a 5,120 x 8,192 product takes 13 % longer with cut tiles than with whole ones)
+            if not swiglu and (offsets is None or 0 < slots <= self.CUT_SLOTS):
                 split_tiles, split = self._k_slices(-(-nout // 16))
                 units = max(slots, 1) * split_tiles
                 if units > self.SLICE_TICKETS or (k + 63) // 64 < split:

@@ -807,7 +807,8 @@ def test_weight_streaming_product_over_group_slots(ops, n, e, nout, k):
                       x[n:].float() @ w_last.float().t()])
     assert float((got - want).abs().max() / want.abs().max()) <= 2e-5
     assert float((every - want).abs().max() / want.abs().max()) <= 2e-5
-    if ops._k_slices(-(-nout // 16))[0] == 0:  # (no tile cut: the same blocks form the same sums)
+    # (tiles are cut only in launches of one or two group slots; with no tile cut the same blocks form the same sums)
+    if ops._k_slices(-(-nout // 16))[0] == 0 or 2 * n > ops.CUT_SLOTS:
         assert torch.equal(got, every)
     # gathered rows, scaled, with the fused activation (the first product of an expert layer)
     h = _rand(n, k, dt=dt, seed=4)
