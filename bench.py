@@ -40,6 +40,8 @@ def main() -> int:
                     help="other decode steps to report: batch or batch@context, comma-separated")
     ap.add_argument("--prefill-points", default="8192", help="other prefill lengths to report")
     ap.add_argument("--point-steps", type=int, default=12)
+    ap.add_argument("--serve", default="", help="requests through the scheduler, e.g. 64x512+128@64 (requests x prompt "
+                    "+ output tokens @ decode batch), comma-separated: tokens a second end to end")
     ap.add_argument("--preset", default="llama4-scout")
     ap.add_argument("--no-prefill", action="store_true")
     args = ap.parse_args()
@@ -171,6 +173,34 @@ def main() -> int:
         s_, frac = run_prefill(T, 2)
         points[f"prefill_{T}"] = round(T / s_, 1)
         points[f"prefill_{T}_frac"] = round(frac, 4)
+
+    # ------------------------------------------------------------------ whole requests through the scheduler
+    for spec in [v for v in args.serve.split(",") if v]:
+        from jax_llm_examples_amd.engine.engine import Engine
+        reqs_s, _, rest = spec.partition("x")
+        plen_s, _, rest = rest.partition("+")
+        olen_s, _, dbs_s = rest.partition("@")
+        nreq, plen, olen = int(reqs_s), int(plen_s), int(olen_s)
+        dbs = int(dbs_s) if dbs_s else min(nreq, 64)
+        eng = Engine(model, cache_tokens=dbs * (plen + olen + 4 * page), decode_batch_size=dbs, page_size=page,
+                     max_num_batched_tokens=2048, max_seq_len=plen + olen + 8)
+        prompts = [torch.randint(0, V, (plen,), generator=gen).tolist() for _ in range(nreq)]
+        # (every other request samples with a temperature; none ends early)
+        sp = [SamplingParams(max_decode_length=olen, sample_temp=0.0 if i % 2 == 0 else 0.8, seed=i, ignore_eos=True)
+              for i in range(nreq)]
+        eng.generate(prompts[:dbs], [SamplingParams(max_decode_length=4, ignore_eos=True)] * min(nreq, dbs))  # records
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        outs = eng.generate(prompts, sp)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t1
+        made = sum(len(o) for o in outs)
+        print(f"[bench] {nreq} requests of {plen} + {olen} tokens, at most {dbs} decoding together: {dt:.2f} s, "
+              f"{made / dt:.0f} generated tok/s, {(made + nreq * plen) / dt:.0f} processed tok/s", file=sys.stderr,
+              flush=True)
+        points[f"serve_{nreq}x{plen}+{olen}_b{dbs}"] = round(made / dt, 1)
+        del eng
+        torch.cuda.empty_cache()
 
     achieved = nbytes["total"] / sec / 1e9
     out = {
