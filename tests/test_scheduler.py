@@ -157,3 +157,20 @@ def test_a_request_ends_at_the_context_limit():
                                                                                 (9, "length")]
     assert max(r.num_computed for r in reqs) <= 30  # no token was ever given a position beyond the limit
     assert cache.num_live() == 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The engine runs on one GPU: ``bench.py --gpus 2`` prints one line that says so and exits with 2."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert p.returncode == 2
+    lines = [ln for ln in p.stdout.splitlines() if ln.strip()]
+    assert len(lines) == 1 and "one GPU" in lines[0]
+    env = dict(os.environ, WORLD_SIZE="2")
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py")], capture_output=True, text=True, timeout=120,
+                       env=env)
+    assert p.returncode == 2
