@@ -524,10 +524,13 @@ class HipOps:
 
     PREFILL_TILE = 32  # tokens per prefill work item (the kernels take 16 or 32)
     GENERIC_SPLIT_BELOW = 2048  # the float32-arithmetic attention: fewer (token, head) pairs than this share their keys
-    DECODE_ITEMS = 1024  # decode attention: work items (wavefronts) that run at once, one per SIMD
-    DECODE_MIN_SPLIT = 128  # keys per work item at least (fewer: the merge costs more than the spreading gains)
-    DECODE_FIT_SPLIT = 1024  # ... at most, to make the items fit in one go
-    DECODE_MAX_SPLIT = 512  # ... when there are more items than fit anyway
+    DECODE_MIN_SPLIT = 128  # decode attention: keys per work item (wavefront) at least ...
+    DECODE_FIT_SPLIT = 1024  # ... and at most
+    DECODE_MAX_SPLIT = 512  # (a step without single tokens: no matter)
+    # measured on MI355X at head size 128 (bfloat16): a block of four wavefronts reads a key position (keys and values
+    # of one kv head) of each in 0.073 us when every compute unit reads; results handed between blocks cost 5.5 us
+    # and 0.09 us per block of the (token, kv head)
+    DECODE_KEY_US, DECODE_MERGE_US, DECODE_RESULT_US = 0.073, 5.5, 0.09
 
     @staticmethod
     def _most_ranges(retention, bound: int, split: int) -> int:
@@ -569,20 +572,25 @@ class HipOps:
                 seg_tiles.append((first, len(tiles) // 2 - first, seg_starts[i] + n - 1))
             o += n
         split, max_splits = self.DECODE_MAX_SPLIT, 1
-        if dec and decode_bucket is not None:
+        if dec:
+            # Which range (a multiple of 32 keys): the one with which the busiest compute unit has the fewest keys
+            # to read.  A block is four ranges of one (token, kv head); a compute unit reads about as fast with
+            # two blocks as with one, so what counts is how many blocks it gets (the blocks over the compute
+            # units, rounded up) times the block's keys; blocks that hand results to each other pay for the merge.
+            if decode_bucket is not None:
+                ranges_of = lambda cand: [self._most_ranges(retention, decode_bucket, cand)] * len(dec)
+            else:
+                ranges_of = lambda cand: [p // cand - f // cand + 1 for f, p in spans]
+            best = None
             for cand in range(self.DECODE_MIN_SPLIT, self.DECODE_FIT_SPLIT + 1, 32):
-                if num_kv_heads * len(dec) * self._most_ranges(retention, decode_bucket, cand) <= self.DECODE_ITEMS:
-                    split = cand
-                    break
-            max_splits = self._most_ranges(retention, decode_bucket, split)
-        elif dec:
-            # the smallest range (a multiple of 32 keys) with which the work items still fit the GPU in one go:
-            # a compute unit that gets a second item beside its first takes much longer than the others
-            for cand in range(self.DECODE_MIN_SPLIT, self.DECODE_FIT_SPLIT + 1, 32):
-                if num_kv_heads * sum(p // cand - f // cand + 1 for f, p in spans) <= self.DECODE_ITEMS:
-                    split = cand
-                    break
-            max_splits = max(p // split - f // split + 1 for f, p in spans)
+                per_unit = [-(-r // 4) for r in ranges_of(cand)]  # blocks per (token, kv head)
+                blocks = num_kv_heads * sum(per_unit)
+                cost = (-(-blocks // self._compute_units) * cand * self.DECODE_KEY_US
+                        + (self.DECODE_MERGE_US + self.DECODE_RESULT_US * max(per_unit) if max(per_unit) > 1 else 0.0))
+                if best is None or cost <= best[0]:  # (equal: the longer range, fewer blocks)
+                    best = (cost, cand)
+            split = best[1]
+            max_splits = max(ranges_of(split))
         groups = []
         if tiles and group_size > 1 and self.PREFILL_TILE == 32:
             # consecutive (tile, head) items of one segment, `waves` per block; blocks with the most keys first
