@@ -1,5 +1,7 @@
 // Router: float32 logits, the k largest per token (lowest index first among equals),
 // gate = sigmoid(logit); and the stable grouping of (token, choice) pairs by expert.
+#include <limits.h>
+
 #include "common.h"
 #include "rows.h"
 
@@ -118,6 +120,54 @@ __device__ __forceinline__ void topk_of_token(const float* __restrict__ logits, 
   }
 #pragma unroll
   for (int j = 0; j < kMaxTopK; ++j) gate[j] = 1.0f / (1.0f + expf(-best_v[j]));
+}
+
+// The same choice made by a whole wavefront for one token, for 64 to 64 * kWaveTopKPerLane experts: every lane
+// fetches its experts' logits at once (expert = lane, lane + 64, ...), then k times the lanes agree on the largest
+// logit not yet taken (the lowest index among equals) with a butterfly of compares.  All lanes return the result.
+constexpr int kWaveTopKPerLane = 4;
+template <bool ACROSS = false>
+__device__ __forceinline__ void topk_of_token_by_wave(const float* __restrict__ logits, size_t n, int E, int k,
+                                                      int (&best_i)[kMaxTopK], float (&gate)[kMaxTopK]) {
+  const int lane = threadIdx.x & 63;
+  float v[kWaveTopKPerLane];
+  bool open[kWaveTopKPerLane];  // an expert of this lane that is not taken yet
+#pragma unroll
+  for (int j = 0; j < kWaveTopKPerLane; ++j) {
+    const int e = lane + 64 * j;
+    open[j] = e < E;
+    v[j] = 0.f;
+    if (open[j]) v[j] = ACROSS ? get_shared(logits + n * E + e) : logits[n * E + e];
+  }
+#pragma unroll
+  for (int r = 0; r < kMaxTopK; ++r) {
+    best_i[r] = -1;
+    gate[r] = 0.f;
+    if (r < k) {
+      float bv = 0.f;
+      int be = INT_MAX;  // (none)
+#pragma unroll
+      for (int j = 0; j < kWaveTopKPerLane; ++j)
+        if (open[j] && (be == INT_MAX || v[j] > bv)) {  // strict '>' keeps the lower index ahead among equals
+          bv = v[j];
+          be = lane + 64 * j;
+        }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oe = __shfl_xor(be, o, 64);
+        if (oe != INT_MAX && (be == INT_MAX || ov > bv || (ov == bv && oe < be))) {
+          bv = ov;
+          be = oe;
+        }
+      }
+      best_i[r] = be;
+      gate[r] = 1.0f / (1.0f + expf(-bv));
+#pragma unroll
+      for (int j = 0; j < kWaveTopKPerLane; ++j)
+        if (be == lane + 64 * j) open[j] = false;
+    }
+  }
 }
 
 __global__ void moe_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids, float* __restrict__ gates,
@@ -394,18 +444,38 @@ __global__ __launch_bounds__(256) void norm_route_kernel(const float* __restrict
   const int M = N * k;
   int* ids_s = ismem + 2 * E + 1;
   float* gates_s = reinterpret_cast<float*>(ids_s + M);
-  const int t = threadIdx.x;
-  if (t < N) {
-    int best_i[kMaxTopK];
-    float gate[kMaxTopK];
-    topk_of_token<true>(logits, (size_t)t, E, k, best_i, gate);
+  if (E >= 64 && E <= 64 * kWaveTopKPerLane) {
+    // many experts: a wavefront per token, the token's logits fetched in one trip
+    for (int t = wave_index(); t < N; t += THREADS / 64) {
+      int best_i[kMaxTopK];
+      float gate[kMaxTopK];
+      topk_of_token_by_wave<true>(logits, (size_t)t, E, k, best_i, gate);
+      if (lane == 0) {
 #pragma unroll
-    for (int j = 0; j < kMaxTopK; ++j) {
-      if (j < k) {
-        ids[t * k + j] = best_i[j];
-        gates[t * k + j] = gate[j];
-        ids_s[t * k + j] = best_i[j];
-        gates_s[t * k + j] = gate[j];
+        for (int j = 0; j < kMaxTopK; ++j) {
+          if (j < k) {
+            ids[t * k + j] = best_i[j];
+            gates[t * k + j] = gate[j];
+            ids_s[t * k + j] = best_i[j];
+            gates_s[t * k + j] = gate[j];
+          }
+        }
+      }
+    }
+  } else {
+    const int t = threadIdx.x;
+    if (t < N) {
+      int best_i[kMaxTopK];
+      float gate[kMaxTopK];
+      topk_of_token<true>(logits, (size_t)t, E, k, best_i, gate);
+#pragma unroll
+      for (int j = 0; j < kMaxTopK; ++j) {
+        if (j < k) {
+          ids[t * k + j] = best_i[j];
+          gates[t * k + j] = gate[j];
+          ids_s[t * k + j] = best_i[j];
+          gates_s[t * k + j] = gate[j];
+        }
       }
     }
   }
