@@ -45,10 +45,29 @@ constexpr int kSkinnyChunks = 4;  // chunks of 32 k on their way per wavefront
 template <bool SWIGLU>
 __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
     const float* __restrict__ X, const float* __restrict__ W, float* __restrict__ Y, const int* __restrict__ offsets,
-    const int* __restrict__ a_rows, const float* __restrict__ scale, int M, int Nout, int K) {
+    const int* __restrict__ a_rows, const float* __restrict__ scale, int M, int Nout, int K, int num_groups,
+    int slots) {
   constexpr int RT = SWIGLU ? 2 : 1;
   __shared__ float red[kSkinnyWaves][RT * 4][64];
-  const int e = blockIdx.z;
+  int e = blockIdx.z;
+  if (slots) {
+    // the blockIdx.z-th group that has rows: 64 groups per look, counted with a ballot
+    const int ln = threadIdx.x & 63;
+    int found = -1, seen = 0;
+    for (int g0 = 0; g0 < num_groups && found < 0; g0 += 64) {
+      const int gi = g0 + ln;
+      const bool has = gi < num_groups && offsets[gi + 1] > offsets[gi];
+      unsigned long long mask = __ballot(has);
+      const int c = __popcll(mask);
+      if ((int)blockIdx.z < seen + c) {
+        for (int j = (int)blockIdx.z - seen; j > 0; --j) mask &= mask - 1;  // drop the lower set bits
+        found = g0 + __ffsll((long long)mask) - 1;
+      }
+      seen += c;
+    }
+    if (found < 0) return;  // fewer groups have rows than there are slots
+    e = __builtin_amdgcn_readfirstlane(found);
+  }
   int row_lo = 0, row_hi = M;
   if (offsets != nullptr) {
     row_lo = offsets[e];
@@ -127,20 +146,26 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
 }  // namespace
 
 // X [*, K], W [G, Nout, K], Y [M, Nout] (or [M, Nout / 2] with swiglu), all float32; K a multiple of 4 and every
-// row 16-byte aligned.  max_rows: the most rows any group can have (M if unknown).
+// row 16-byte aligned.  max_rows: the most rows any group can have (M if unknown).  slots > 0: only so many groups
+// can have rows (there are no more rows than that): the launch has that many group slots instead of G groups
+// (slot j works on the j-th group that has rows) - with few rows over many groups most blocks of a launch over all
+// groups would only start and leave, and the launch takes as long as starting its wavefronts takes.
 JLE_API int jle_gemm_f32_skinny(const float* X, const float* W, float* Y, const int* offsets, const int* a_rows,
                                 const float* scale, int swiglu, int M, int Nout, int K, int G, int max_rows,
-                                hipStream_t s) {
+                                int slots, hipStream_t s) {
   if (M <= 0 || Nout <= 0) return 0;
   if (K <= 0 || K % 4 || G < 1 || G > 65535 || (swiglu && Nout % 2)) return JLE_BAD_ARG;
+  if (slots < 0 || (slots > 0 && (offsets == nullptr || slots > G))) return JLE_BAD_ARG;
   if ((((uintptr_t)X | (uintptr_t)W | (uintptr_t)Y) & 15) != 0) return JLE_BAD_ARG;
   if (max_rows <= 0 || max_rows > M) max_rows = M;
   const int cols = swiglu ? Nout / 2 : Nout;
   const int ytiles = (max_rows + 15) / 16;
   if (ytiles > 65535) return JLE_BAD_ARG;
-  dim3 g((cols + 15) / 16, ytiles, offsets != nullptr ? G : 1), b(kSkinnyWaves * 64);
-  if (swiglu) hipLaunchKernelGGL(gemm_f32_skinny_kernel<true>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);
-  else hipLaunchKernelGGL(gemm_f32_skinny_kernel<false>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K);
+  dim3 g((cols + 15) / 16, ytiles, offsets != nullptr ? (slots > 0 ? slots : G) : 1), b(kSkinnyWaves * 64);
+  if (swiglu)
+    hipLaunchKernelGGL(gemm_f32_skinny_kernel<true>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K, G, slots);
+  else
+    hipLaunchKernelGGL(gemm_f32_skinny_kernel<false>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K, G, slots);
   JLE_LAUNCH_CHECK();
   return 0;
 }

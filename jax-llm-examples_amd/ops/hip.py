@@ -45,7 +45,7 @@ _SIGNATURES = {
     "jle_moe_align": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "jle_moe_route_align": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-    "jle_gemm_f32_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_f32_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
     "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
@@ -298,8 +298,10 @@ class HipOps:
             raise KernelError(f"the float32 matrix-core product needs an inner size that is a multiple of 4 and "
                               f"16-byte aligned rows, got K = {k}")
         out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32, device=a.device)
+        # (no more groups have rows than there are rows: so many group slots instead of every group)
+        slots = m if offsets is not None and g > m else 0
         self._call("jle_gemm_f32_skinny", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu), m,
-                   nout, k, g, m)
+                   nout, k, g, m, slots)
         return out
 
     SKINNY_MAX_ROWS = 64  # up to here a product is a stream of the weights: the MFMA weight-streaming kernel
