@@ -71,7 +71,7 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_reg_kernel(float* __restr
 // Rows whose width is a multiple of 8 (and 16-byte aligned arrays): a thread takes CPT pieces of 4
 // neighbouring elements, piece = thread, thread + THREADS, ...; up to THREADS * CPT * 4 wide.
 template <typename DT, typename OT, int THREADS, int CPT, bool STREAM>
-__global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ x, Delta<DT> delta,
+__global__ __launch_bounds__(THREADS, 4) void add_rmsnorm_vec_kernel(float* __restrict__ x, Delta<DT> delta,
                                                                   const float* __restrict__ w, float eps,
                                                                   OT* __restrict__ out, float* __restrict__ out32,
                                                                   int D) {
@@ -88,23 +88,33 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
   f32x4_t v[CPT];
   float ss = 0.f;
   const bool add = delta.any();
+  const DeltaRow<DT> drow = delta_row(delta, n, D);
 #pragma unroll
   for (int i = 0; i < CPT; ++i) {
     const int d = (threadIdx.x + THREADS * i) * 4;
-    v[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    if (d < D) {
-      v[i] = load4_as<STREAM, float>(x + base + d);
-      if (add) {
-        v[i] += delta_at4<STREAM, DT>(delta, n, d, D);
+    v[i] = d < D ? load4_as<STREAM, float>(x + base + d) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  // (every load before the first store: a store in between would make the loads after it wait, since the
+  // compiler cannot know that x is none of the arrays they read.  The pieces past the row's end are selects,
+  // not branches around an update of v[i]: with those the compiler carries the whole array as one wide value
+  // and needs 211 registers instead of 118, which halves the rows a compute unit works on at once.)
+  if (add) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int d = (threadIdx.x + THREADS * i) * 4;
+      v[i] += d < D ? delta_row_at4<STREAM, DT>(delta, drow, n, d, D) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int d = (threadIdx.x + THREADS * i) * 4;
+      if (d < D) {
         if (STREAM) __builtin_nontemporal_store(v[i], reinterpret_cast<f32x4_t*>(x + base + d));
         else store4<float>(x + base + d, v[i]);
       }
-      ss += v[i][0] * v[i][0];
-      ss += v[i][1] * v[i][1];
-      ss += v[i][2] * v[i][2];
-      ss += v[i][3] * v[i][3];
     }
   }
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) ss = add_squares4(ss, v[i]);
   const float tot = block_sum<THREADS>(ss, red);
   const float inv = 1.0f / sqrtf(tot / (float)D + eps);
 #pragma unroll

@@ -366,20 +366,29 @@ __global__ __launch_bounds__(256) void norm_route_kernel(const float* __restrict
   f32x4_t v[CPT];
   float ss = 0.f;
   const bool add = delta.any();
+  const DeltaRow<DT> drow = delta_row(delta, n, D);
 #pragma unroll
   for (int i = 0; i < CPT; ++i) {
     const int d = (threadIdx.x + THREADS * i) * 4;
-    v[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    if (d < D) {
-      v[i] = load4<float>(x + base + d);
-      if (add) v[i] += delta_at4<false, DT>(delta, n, d, D);
-      if (writer) store4<float>(x_out + base + d, v[i]);
-      ss += v[i][0] * v[i][0];
-      ss += v[i][1] * v[i][1];
-      ss += v[i][2] * v[i][2];
-      ss += v[i][3] * v[i][3];
+    v[i] = d < D ? load4<float>(x + base + d) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  // (every load before the first store: see add_rmsnorm_vec_kernel)
+  if (add) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int d = (threadIdx.x + THREADS * i) * 4;
+      v[i] += d < D ? delta_row_at4<false, DT>(delta, drow, n, d, D) : f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
   }
+  if (writer) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int d = (threadIdx.x + THREADS * i) * 4;
+      if (d < D) store4<float>(x_out + base + d, v[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) ss = add_squares4(ss, v[i]);
   const float tot = block_sum<THREADS>(ss, red);
   const float rs = 1.0f / sqrtf(tot / (float)D + eps);
 #pragma unroll

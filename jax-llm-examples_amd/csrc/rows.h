@@ -79,6 +79,7 @@ __device__ __forceinline__ f32x4_t delta_at4(const Delta<DT>& delta, size_t n, i
   f32x4_t v = {0.f, 0.f, 0.f, 0.f};
   if (delta.plain != nullptr) v = load4_as<STREAM, DT>(delta.plain + n * D + d);
   if (delta.routed != nullptr) {
+#pragma nounroll
     for (int j = 0; j < delta.k; ++j)
       v += load4_as<STREAM, DT>(delta.routed + (size_t)delta.inv[n * delta.k + j] * D + d);
     if (delta.shared != nullptr) v += load4_as<STREAM, DT>(delta.shared + n * D + d);
@@ -86,5 +87,48 @@ __device__ __forceinline__ f32x4_t delta_at4(const Delta<DT>& delta, size_t n, i
   return v;
 }
 
+// What a row's delta is made of, looked up once per row: for a plain tensor and for tokens with one expert the
+// row(s) to read; tokens with several experts keep the general sum (delta_at4), piece by piece.
+template <typename DT>
+struct DeltaRow {
+  const DT* a;      // the plain row, or the row of the token's one expert
+  const DT* b;      // the shared expert's row, or null
+  bool from_zero;   // a is an expert's row: the sum starts from zero, as delta_at4's does
+  bool general;
+};
+template <typename DT>
+__device__ __forceinline__ DeltaRow<DT> delta_row(const Delta<DT>& delta, size_t n, int D) {
+  DeltaRow<DT> r = {nullptr, nullptr, false, false};
+  if (delta.plain != nullptr && delta.routed == nullptr) {
+    r.a = delta.plain + n * D;
+  } else if (delta.plain == nullptr && delta.routed != nullptr && delta.k == 1) {
+    r.a = delta.routed + (size_t)delta.inv[n] * D;
+    r.b = delta.shared != nullptr ? delta.shared + n * D : nullptr;
+    r.from_zero = true;
+  } else {
+    r.general = true;
+  }
+  return r;
+}
+template <bool STREAM, typename DT>
+__device__ __forceinline__ f32x4_t delta_row_at4(const Delta<DT>& delta, const DeltaRow<DT>& row, size_t n, int d,
+                                                 int D) {
+  if (row.general) return delta_at4<STREAM, DT>(delta, n, d, D);
+  f32x4_t v = load4_as<STREAM, DT>(row.a + d);
+  if (row.from_zero) v = f32x4_t{0.f, 0.f, 0.f, 0.f} + v;
+  if (row.b != nullptr) v += load4_as<STREAM, DT>(row.b + d);
+  return v;
+}
+
+// ss + the squares of four neighbours, one fused multiply-add after the other in this order: written out, since the
+// compiler, left to fuse "ss += a * a" itself, may pick another order in another kernel, and the kernels that norm
+// a row have to agree to the bit.
+__device__ __forceinline__ float add_squares4(float ss, f32x4_t v) {
+  ss = __builtin_fmaf(v[0], v[0], ss);
+  ss = __builtin_fmaf(v[1], v[1], ss);
+  ss = __builtin_fmaf(v[2], v[2], ss);
+  ss = __builtin_fmaf(v[3], v[3], ss);
+  return ss;
+}
 
 }  // namespace jle
