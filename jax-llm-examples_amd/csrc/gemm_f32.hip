@@ -1,6 +1,6 @@
-// Grouped weight-streaming matrix product in true float32 on the matrix cores (v_mfma_f32_16x16x4_f32: float32
+// Grouped weight-streaming matrix products in true float32 on the matrix cores (v_mfma_f32_16x16x4_f32: float32
 // operands, float32 products and sums; no reduced-precision mode anywhere): what the float32 run of the model
-// uses for its routed experts in steps of few tokens.
+// uses for its routed experts, one kernel for steps of few tokens, one for a prefill's hundred rows per expert.
 //
 //   Y[t, n] = scale[t] * sum_k X[arow(t), k] * W[g(t)][n, k]                         (plain)
 //   Y[t, f] = silu(s * gate) * (s * up), gate / up = rows f and F + f of W[g(t)]      (SWIGLU)
@@ -10,9 +10,10 @@
 //
 // Few rows (decode; a group's rows in tiles of 16): the cost is reading W once.  The weights are the A operand,
 // the tokens' rows the B operand.  The wavefronts of a block split K (every 8th chunk of 32 k each) and add their
-// sums in shared memory in a fixed order.  (With many rows per group the general float32 kernel of
-// gemm_generic.hip is the faster one: a 128 x 128 x 32 tiled kernel on these instructions reached 44 to 63
-// TFLOP/s at 128 to 512 rows per expert where that one reaches 58 to 70, and was taken out again.)
+// sums in shared memory in a fixed order.  Many rows per group: further down.  (A 128 x 128 x 32 kernel with both
+// operands tiled through shared memory reached 44 to 63 TFLOP/s on these instructions at 128 to 512 rows per
+// expert, where the general float32 kernel of gemm_generic.hip reaches 58 to 70, and was taken out again; the
+// kernel below, whose weights never pass through shared memory, reaches 84 to 114.)
 //
 // Order of the sums: an element's sum over k is formed per wavefront over its chunks in ascending order, within
 // a chunk in the order of the instruction's 4 k-lanes and the lane's 8 elements; the wavefronts' sums are added
@@ -143,6 +144,187 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
   else Y[(size_t)t * Nout + col] = v0 * sc;
 }
 
+// ------------------------------------------------------------------------------------------ about a hundred rows
+// A prefill's rows per expert (around a hundred): every element of W should be read once, so a wavefront owns two
+// 16-row tiles of W (SWIGLU: a gate tile and its up tile) and up to 192 rows of its group, as gemm_stream.hip does
+// for bfloat16: the weights go from memory straight into the A operands (a lane's 8 consecutive floats of its row
+// feed 8 instructions, as above), the rows of X are shared by the block's wavefronts through shared memory, 32 k
+// at a time (rows 144 bytes apart: the 16 lanes of an instruction's k-lane read 16 rows without meeting in a
+// bank).  A stage's weights and rows are asked for two stages ahead (a stage is thousands of cycles of arithmetic:
+// longer than a trip to memory).  K must be a multiple of 64 (whole rounds of two stages).  Groups with more than 192 rows are done in passes (each reads the weights again).
+// The arithmetic is the limit here (each instruction is 2,048 operations in 32 cycles of a SIMD), not the stream.
+//
+// Order of the sums: over the stages in ascending order, within a stage as in the kernel above; it depends on K
+// only.
+constexpr int kStreamRows = 192;  // rows of a pass
+constexpr int SBK = 32;           // k per stage
+constexpr int SPITCH = 36;        // floats from row to row in shared memory
+constexpr int kStreamWaves = 8;
+
+template <bool SWIGLU, int NTL>
+__device__ __forceinline__ void f32_stream_block(const float* __restrict__ X, const float* __restrict__ w0,
+                                                 const float* __restrict__ w1, float* __restrict__ Y,
+                                                 const int* __restrict__ a_rows, const float* __restrict__ scale,
+                                                 float (&sX)[2][kStreamRows * SPITCH], int tok0, int live, int K,
+                                                 int Nout, int c0, int c1, bool wave_ok) {
+  constexpr int THREADS = kStreamWaves * 64;
+  constexpr int CHUNKS = NTL * 16 * (SBK / 4);            // 16-byte pieces of X per stage
+  constexpr int CPT = (CHUNKS + THREADS - 1) / THREADS;  // per thread
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int nstage = K / SBK;  // a multiple of 2
+  // who brings which pieces of X: piece c is 4 k of row c / 8
+  uint32_t xsrc[CPT];  // elements from X (the host checks that X has fewer than 2^32)
+  int xdst[CPT];
+#pragma unroll
+  for (int i = 0; i < CPT; ++i) {
+    const int c = threadIdx.x + THREADS * i;
+    const int row = (c >> 3) % kStreamRows, kc = c & 7;  // (past the buffer only if CHUNKS is no multiple of THREADS)
+    const int t = row < live ? tok0 + row : tok0;
+    xsrc[i] = (uint32_t)(a_rows != nullptr ? a_rows[t] : t) * (uint32_t)K + kc * 4;
+    xdst[i] = row * SPITCH + kc * 4;
+  }
+  const int b_off = r * SPITCH + 8 * g;  // this lane's 8 floats of row r of a tile of rows
+
+  f32x4 acc0[NTL], acc1[NTL];
+#pragma unroll
+  for (int nt = 0; nt < NTL; ++nt) {
+    acc0[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc1[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  f32x4 xr[2][CPT], wr[2][2][2];  // on their way: the pieces of X and the weights [tile][half] of two stages
+  auto ask_rows = [&](f32x4 (&x)[CPT], int s) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) x[i] = *reinterpret_cast<const f32x4*>(X + xsrc[i] + (size_t)s * SBK);
+  };
+  auto ask_weights = [&](f32x4 (&w)[2][2], int s) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      w[0][h] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(w0 + (size_t)s * SBK + 4 * h));
+      w[1][h] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(w1 + (size_t)s * SBK + 4 * h));
+    }
+  };
+  auto put = [&](const f32x4 (&x)[CPT], float* buf) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) *reinterpret_cast<f32x4*>(buf + xdst[i]) = x[i];
+  };
+  auto work = [&](const f32x4 (&w)[2][2], const float* buf) {
+    // (the next tile's rows are read while this tile's 16 instructions run, and no further ahead: left to itself
+    // the compiler reads all tiles' rows first and runs out of registers)
+    f32x4 blo = *reinterpret_cast<const f32x4*>(buf + b_off);
+    f32x4 bhi = *reinterpret_cast<const f32x4*>(buf + b_off + 4);
+#pragma unroll
+    for (int nt = 0; nt < NTL; ++nt) {
+      f32x4 nlo = blo, nhi = bhi;
+      if (nt + 1 < NTL) {
+        nlo = *reinterpret_cast<const f32x4*>(buf + (nt + 1) * 16 * SPITCH + b_off);
+        nhi = *reinterpret_cast<const f32x4*>(buf + (nt + 1) * 16 * SPITCH + b_off + 4);
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float b = h == 0 ? blo[j] : bhi[j];
+          acc0[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[0][h][j], b, acc0[nt], 0, 0, 0);
+          acc1[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[1][h][j], b, acc1[nt], 0, 0, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      blo = nlo;
+      bhi = nhi;
+    }
+  };
+#define STAGE(x_, w_, buf_, s_, ASKX, ASKW)   \
+  do {                                        \
+    put(x_, sX[buf_]);                        \
+    __syncthreads();                          \
+    if (ASKX) ask_rows(x_, (s_) + 2);         \
+    __builtin_amdgcn_sched_barrier(0);        \
+    work(w_, sX[buf_]);                       \
+    if (ASKW) ask_weights(w_, (s_) + 2);      \
+  } while (0)
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    ask_weights(wr[j], j);
+    ask_rows(xr[j], j);
+  }
+  int s = 0;
+  for (; s < nstage - 2; s += 2) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) STAGE(xr[j], wr[j], j, s + j, true, true);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) STAGE(xr[j], wr[j], j, s + j, false, false);
+#undef STAGE
+  if (!wave_ok) return;
+  // accumulators: element i of tile nt in lane (g, r) = weight row 4 g + i of the tile, row 16 nt + r of the pass
+  const int half = Nout >> 1;
+#pragma unroll
+  for (int nt = 0; nt < NTL; ++nt) {
+    const int row = nt * 16 + r;
+    if (row >= live) continue;
+    const int t = tok0 + row;
+    const float sc = scale != nullptr ? scale[t] : 1.f;
+    if (SWIGLU) {
+      f32x4 y;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = silu_mul(acc0[nt][i] * sc, acc1[nt][i] * sc);
+      *reinterpret_cast<f32x4*>(Y + (size_t)t * half + c0 + 4 * g) = y;
+    } else {
+      *reinterpret_cast<f32x4*>(Y + (size_t)t * Nout + c0 + 4 * g) = acc0[nt] * sc;
+      if (c1 != c0) *reinterpret_cast<f32x4*>(Y + (size_t)t * Nout + c1 + 4 * g) = acc1[nt] * sc;
+    }
+  }
+}
+
+template <bool SWIGLU>
+__global__ __launch_bounds__(kStreamWaves * 64, 2) void gemm_f32_stream_kernel(
+    const float* __restrict__ X, const float* __restrict__ W, float* __restrict__ Y, const int* __restrict__ offsets,
+    const int* __restrict__ a_rows, const float* __restrict__ scale, int M, int Nout, int K, int nblk, int passes) {
+  __shared__ __attribute__((aligned(16))) float sX[2][kStreamRows * SPITCH];
+  const int item = blockIdx.x;
+  const int nb = item % nblk, pass = (item / nblk) % passes, e = item / (nblk * passes);
+  int row_lo = 0, row_hi = M;
+  if (offsets != nullptr) {
+    row_lo = offsets[e];
+    row_hi = offsets[e + 1];
+  }
+  const int tok0 = row_lo + pass * kStreamRows;
+  if (tok0 >= row_hi) return;  // the whole block
+  const int live = min(kStreamRows, row_hi - tok0);
+  const int lane = threadIdx.x & 63, wave = wave_index();
+  const int r = lane & 15, g = lane >> 4;
+  const int half = Nout >> 1;
+  const float* We = W + (size_t)e * Nout * K;
+  // the wavefront's two weight tiles: first columns c0 and c1 of the output
+  const int ntile = (SWIGLU ? half : Nout) >> 4;
+  int c0, c1, row1;
+  bool wave_ok;
+  if (SWIGLU) {
+    const int ft = nb * kStreamWaves + wave;
+    wave_ok = ft < ntile;
+    c0 = (wave_ok ? ft : 0) * 16;
+    c1 = c0;
+    row1 = half + c0;
+  } else {
+    const int ft = (nb * kStreamWaves + wave) * 2;
+    wave_ok = ft < ntile;
+    c0 = (wave_ok ? ft : 0) * 16;
+    c1 = min(c0 + 16, (ntile - 1) * 16);
+    row1 = c1;
+  }
+  const float* w0 = We + (size_t)(c0 + r) * K + 8 * g;
+  const float* w1 = We + (size_t)(row1 + r) * K + 8 * g;
+#define GO(NTL_) f32_stream_block<SWIGLU, NTL_>(X, w0, w1, Y, a_rows, scale, sX, tok0, live, K, Nout, c0, c1, wave_ok)
+  if (live <= 32) GO(2);
+  else if (live <= 64) GO(4);
+  else if (live <= 96) GO(6);
+  else if (live <= 128) GO(8);
+  else if (live <= 160) GO(10);
+  else GO(12);
+#undef GO
+}
+
 }  // namespace
 
 // X [*, K], W [G, Nout, K], Y [M, Nout] (or [M, Nout / 2] with swiglu), all float32; K a multiple of 4 and every
@@ -166,6 +348,38 @@ JLE_API int jle_gemm_f32_skinny(const float* X, const float* W, float* Y, const 
     hipLaunchKernelGGL(gemm_f32_skinny_kernel<true>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K, G, slots);
   else
     hipLaunchKernelGGL(gemm_f32_skinny_kernel<false>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K, G, slots);
+  JLE_LAUNCH_CHECK();
+  return 0;
+}
+
+// Whether jle_gemm_f32_stream takes these sizes.
+JLE_API int jle_gemm_f32_stream_supported(int Nout, int K, int swiglu) {
+  if (K <= 0 || K % (SBK * 2)) return 0;
+  if (swiglu) return Nout > 0 && Nout % 32 == 0;
+  return Nout > 0 && Nout % 16 == 0;
+}
+
+// The same product for about a hundred rows per group (see the kernel): X must have its rows 16-byte aligned, K a
+// multiple of 64, whole tiles of 16 weight rows (32 with swiglu), X fewer than 2^32 elements.  max_rows: the most rows any group can have
+// (M if unknown).
+JLE_API int jle_gemm_f32_stream(const float* X, const float* W, float* Y, const int* offsets, const int* a_rows,
+                                const float* scale, int swiglu, int M, int Nout, int K, int G, int max_rows,
+                                hipStream_t s) {
+  if (M <= 0 || Nout <= 0) return 0;
+  if (G < 1 || G > 65535 || !jle_gemm_f32_stream_supported(Nout, K, swiglu)) return JLE_BAD_ARG;
+  if ((((uintptr_t)X | (uintptr_t)W | (uintptr_t)Y) & 15) != 0) return JLE_BAD_ARG;
+  if (max_rows <= 0 || max_rows > M) max_rows = M;
+  const int passes = (max_rows + kStreamRows - 1) / kStreamRows;
+  const int pairs = swiglu ? Nout / 32 : (Nout / 16 + 1) / 2;  // pairs of weight tiles = wavefronts needed per group
+  const int nblk = (pairs + kStreamWaves - 1) / kStreamWaves;
+  if ((long long)nblk * passes * G > (1ll << 30)) return JLE_BAD_ARG;
+  const dim3 grid(nblk * passes * G), block(kStreamWaves * 64);
+  if (swiglu)
+    hipLaunchKernelGGL(gemm_f32_stream_kernel<true>, grid, block, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K,
+                       nblk, passes);
+  else
+    hipLaunchKernelGGL(gemm_f32_stream_kernel<false>, grid, block, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K,
+                       nblk, passes);
   JLE_LAUNCH_CHECK();
   return 0;
 }

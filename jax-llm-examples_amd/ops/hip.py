@@ -46,6 +46,7 @@ _SIGNATURES = {
     "jle_moe_route_align": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_generic": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_gemm_f32_skinny": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "jle_gemm_f32_stream": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "jle_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "jle_attention_mfma_supported": [_i, _i, _i, _i],
     "jle_attention_prefill": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _i, _i, _i, _vp],
@@ -120,6 +121,7 @@ def load_library():
             fn.restype = ctypes.c_int
         lib.jle_attention_mfma_supported.argtypes = [_i, _i, _i, _i]  # a query, not a launch: no stream
         lib.jle_gemm_stream_supported.argtypes = [_i, _i, _i]
+        lib.jle_gemm_f32_stream_supported.argtypes = [_i, _i, _i]
         lib.jle_attention_group_waves.argtypes = []
         lib._jle_path = path
         _LIB = lib
@@ -279,8 +281,9 @@ class HipOps:
                    1 if (out_f32 or a.dtype == torch.float32) else 0, m, nout, k, g)
         return out
 
-    F32_SKINNY_ROWS = 128  # float32 grouped products: up to so many rows the weight-streaming kernel on the float32
-    # matrix instructions; beyond, the general kernel (measured faster there than a tiled kernel on those instructions)
+    F32_SKINNY_ROWS = 128  # float32 grouped products: up to so many rows (of all groups together) the kernel whose
+    # wavefronts split K; beyond, the one whose wavefronts hold up to 192 rows of a group (both on the float32 matrix
+    # instructions); the general kernel where the sizes do not fit either
 
     def gemm_f32_skinny(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, rows=None):
         """The float32 grouped product for few rows on the float32 matrix instructions (see ``gemm_f32.hip``):
@@ -302,6 +305,31 @@ class HipOps:
         slots = m if offsets is not None and g > m else 0
         self._call("jle_gemm_f32_skinny", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu), m,
                    nout, k, g, m, slots)
+        return out
+
+    def f32_stream_supported(self, nout: int, k: int, swiglu: bool) -> bool:
+        return bool(self.lib.jle_gemm_f32_stream_supported(nout, k, int(swiglu)))
+
+    def gemm_f32_stream(self, a, b, *, offsets=None, a_rows=None, scale=None, swiglu=False, rows=None):
+        """The float32 grouped product for about a hundred rows per group on the float32 matrix instructions,
+        the weights read once per 192 rows of a group (see ``gemm_f32.hip``)."""
+        if b.dim() == 2:
+            b = b.unsqueeze(0)
+        g, nout, k = b.shape
+        m = rows if rows is not None else (a_rows.numel() if a_rows is not None else a.shape[0])
+        self._chk(a, torch.float32, None, "A")
+        self._chk(b, torch.float32, None, "B")
+        if a.shape[1] != k:
+            raise KernelError(f"inner sizes differ: A {tuple(a.shape)}, B {tuple(b.shape)}")
+        if a.numel() >= 2 ** 32:
+            raise KernelError("the float32 weight-streaming grouped product addresses its rows with 32 bits")
+        if not self.f32_stream_supported(nout, k, swiglu) or a.data_ptr() % 16 or b.data_ptr() % 16:
+            raise KernelError(f"the float32 weight-streaming grouped product needs an inner size that is a multiple of "
+                              f"64, whole tiles of 16 weight rows (32 with the fused activation) and 16-byte aligned "
+                              f"rows, got {nout} x {k}")
+        out = torch.empty(m, nout // 2 if swiglu else nout, dtype=torch.float32, device=a.device)
+        self._call("jle_gemm_f32_stream", _p(a), _p(b), _p(out), _p(offsets), _p(a_rows), _p(scale), int(swiglu), m,
+                   nout, k, g, m)
         return out
 
     SKINNY_MAX_ROWS = 64  # up to here a product is a stream of the weights: the MFMA weight-streaming kernel
@@ -877,6 +905,14 @@ class HipOps:
             act = self.gemm_f32_skinny(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate,
                                        swiglu=True)
             routed = self.gemm_f32_skinny(act, w_down, offsets=offsets)
+        elif (h.dtype == torch.float32 and self.f32_stream_supported(f2, d, True)
+              and self.f32_stream_supported(d, f2 // 2, False) and h.numel() < 2 ** 32 and m * (f2 // 2) < 2 ** 32
+              and not (h.data_ptr() | w_gate_up.data_ptr() | w_down.data_ptr()) % 16):
+            # more rows in true float32 (a prefill): the same instructions, a wavefront holding up to 192 rows of
+            # its expert, so that the weights are read once per so many rows
+            act = self.gemm_f32_stream(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate,
+                                       swiglu=True)
+            routed = self.gemm_f32_stream(act, w_down, offsets=offsets)
         else:
             gu = self.gemm(h, w_gate_up, offsets=offsets, a_rows=sorted_token, scale=sorted_gate)
             act = self.silu_mul(gu)

@@ -719,6 +719,61 @@ def test_float32_grouped_product_on_the_float32_matrix_instructions(ops, n, d, f
         ops.gemm_f32_skinny(h[:, : d - 2].contiguous(), wgu[:, :, : d - 2].contiguous())
 
 
+@pytest.mark.parametrize("n,d,f,e,k", [(1, 64, 64, 4, 1), (50, 128, 64, 4, 1), (300, 192, 128, 3, 2), (700, 64, 192, 5, 1),
+                                       (450, 320, 64, 2, 1), (2100, 5120, 128, 16, 1), (200, 1088, 448, 128, 2)])
+def test_float32_grouped_product_for_many_rows_on_the_float32_matrix_instructions(ops, n, d, f, e, k):
+    """The float32 product whose wavefronts hold up to 192 rows of a group (gemm_f32.hip) against float64: grouped,
+    gathered, scaled, with and without the fused activation; groups of more than 192 rows (several passes), of a
+    few rows and of none, rows that fill no tile."""
+    h = _rand(n, d, seed=1)
+    wgu, wd = _rand(e, 2 * f, d, scale=0.1, seed=2), _rand(e, d, f, scale=0.1, seed=3)
+    g = torch.Generator().manual_seed(n)
+    ids = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(n)]).to(torch.int32).to(DEV)
+    if e > 2:
+        ids[ids == 1] = 2  # a group without rows, and one with twice its share
+    gates = torch.rand(n, k, generator=g).to(DEV)
+    off, tok, gate, inv = ops.moe_align(ids, gates, e)
+    act = ops.gemm_f32_stream(h, wgu, offsets=off, a_rows=tok, scale=gate, swiglu=True)
+    gu = ops.gemm_f32_stream(h, wgu, offsets=off, a_rows=tok, scale=gate)
+    sorted_ids = ids.flatten()[torch.argsort(inv.long())].long()
+    x64 = h.double()[tok.long()] * gate.double()[:, None]
+    want_gu = torch.empty(tok.numel(), 2 * f, dtype=torch.float64, device=DEV)
+    for j in range(e):
+        rows = sorted_ids == j
+        want_gu[rows] = x64[rows] @ wgu[j].double().t()
+    want_act = torch.nn.functional.silu(want_gu[:, :f]) * want_gu[:, f:]
+    assert float((gu.double() - want_gu).abs().max() / want_gu.abs().max()) <= 3e-6
+    assert float((act.double() - want_act).abs().max() / want_act.abs().max()) <= 3e-6
+    out = ops.gemm_f32_stream(act, wd, offsets=off)
+    want = torch.empty(tok.numel(), d, dtype=torch.float64, device=DEV)
+    for j in range(e):
+        rows = sorted_ids == j
+        want[rows] = act.double()[rows] @ wd[j].double().t()
+    assert float((out.double() - want).abs().max() / want.abs().max()) <= 3e-6
+    # one group without offsets, and the result of a row does not depend on what else is in the launch
+    # (measured against the sum of the terms' sizes, as for the dense projections above: the sums over 5,120 terms
+    # are formed one stage after the other)
+    dense = ops.gemm_f32_stream(h, wgu[0])
+    terms = h.double().abs() @ wgu[0].double().abs().t()
+    assert float(((dense.double() - h.double() @ wgu[0].double().t()).abs() / terms).max()) < 2e-6
+    assert torch.equal(ops.gemm_f32_stream(h[:1].contiguous(), wgu[0]), dense[:1])
+    with pytest.raises(Exception, match="multiple of 64"):
+        ops.gemm_f32_stream(h[:, : d - 32].contiguous(), wgu[:, :, : d - 32].contiguous())
+    # through the experts' entry: more rows than the few-rows kernel takes
+    if n * k > ops.F32_SKINNY_ROWS:
+        calls = []
+        inner = ops._call
+        ops._call = lambda name, *a: (calls.append(name), inner(name, *a))[1]
+        try:
+            got = ops.materialize(ops.moe_experts(h, ids, gates, wgu, wd, None))
+        finally:
+            ops._call = inner
+        assert calls.count("jle_gemm_f32_stream") == 2, calls
+        want_sum = torch.zeros(n, d, dtype=torch.float64, device=DEV)
+        want_sum.index_add_(0, tok.long(), want)
+        assert float((got.double() - want_sum).abs().max() / want_sum.abs().max()) <= 3e-6
+
+
 def test_sampling(ops, ref):
     g = torch.Generator().manual_seed(0)
     V = 1000
