@@ -38,11 +38,17 @@ __device__ __forceinline__ float4 load_once(const float* p) {
 constexpr int kSkinnyWaves = 8;
 constexpr int kSkinnyChunks = 4;  // chunks of 32 k on their way per wavefront
 
-// A lane reads 8 consecutive floats of its weight row (two 16-byte loads; the 4 lanes of a row read one whole
-// 128-byte line between them, a wavefront 16 rows x 32 k), which feed 8 instructions; the lane of the B operand
-// reads the same 8 k of its token's row.  (Dealing the lanes so that every single load instruction covers whole
-// lines - 8 rows x 128 bytes, the even and the odd 16-byte pieces of a row multiplied in instructions of their
-// own - was measured slower: 805 + 442 us a layer against 622 + 286 for Scout's experts at batch 8.)
+// A lane's A operands are 8 consecutive floats of its weight row (row r = lane % 16, k = 8 g .. 8 g + 7 of the
+// chunk, g = lane / 16), which feed 8 instructions; the lane of the B operand reads the same 8 k of its token's
+// row.  Loaded that way, neighbouring lanes would read from different rows, 20 KB apart, and every lane's 16
+// bytes would be a request of its own to the first-level cache, which takes one a cycle: 17 GB/s a compute unit,
+// what this kernel reached at first (3.5 TB/s).  So a load instruction reads whole 128-byte lines, 8 lanes a
+// row's line, 8 rows, and the lines are turned into the operands' order through a piece of shared memory of the
+// wavefront's own (rows 144 bytes apart: neither writing nor reading collides).  The same products in the same
+// order, so not a bit of the result changes.  (Dealing the lanes so that a line's even and odd 16-byte pieces
+// are multiplied in instructions of their own, without shared memory, was measured slower: twice the
+// instructions.)
+constexpr int kTurnPitch = 36;  // floats from row to row of a wavefront's piece of shared memory
 template <bool SWIGLU>
 __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
     const float* __restrict__ X, const float* __restrict__ W, float* __restrict__ Y, const int* __restrict__ offsets,
@@ -50,6 +56,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
     int slots) {
   constexpr int RT = SWIGLU ? 2 : 1;
   __shared__ float red[kSkinnyWaves][RT * 4][64];
+  __shared__ __attribute__((aligned(16))) float turn[kSkinnyWaves][RT][16 * kTurnPitch];
   int e = blockIdx.z;
   if (slots) {
     // the blockIdx.z-th group that has rows: 64 groups per look, counted with a ballot
@@ -82,9 +89,18 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
   const int half = Nout >> 1;
   const int base = blockIdx.x * 16;  // first output column of the block
   const int cols = SWIGLU ? half : Nout;
-  const int wrow0 = min(base + r, cols - 1);
-  const float* w0 = We + (size_t)wrow0 * K + 8 * g;
-  const float* w1 = We + (size_t)(wrow0 + half) * K + 8 * g;  // (SWIGLU: the up row of the gate row)
+  // what this lane loads: 16 bytes (piece lc) of the lines of rows lr and lr + 8 of the tile
+  const int lr = lane >> 3, lc = lane & 7;
+  const float* wl0[2];
+  const float* wl1[2];  // (SWIGLU: the up row of the gate row)
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int wrow = min(base + 8 * h + lr, cols - 1);
+    wl0[h] = We + (size_t)wrow * K + 4 * lc;
+    wl1[h] = We + (size_t)(wrow + half) * K + 4 * lc;
+  }
+  float* buf0 = turn[wave][0];
+  float* buf1 = turn[wave][RT - 1];
   const int t = tok0 + r;
   const bool xv = t < row_hi;
   const float* xb = X + (size_t)(xv ? (a_rows != nullptr ? a_rows[t] : t) : 0) * K + 8 * g;
@@ -97,21 +113,36 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
     for (int u = 0; u < kSkinnyChunks; ++u) {
       const int c = c0 + kSkinnyWaves * u;
       const int k = c * 32 + 8 * g;
-      // K is a multiple of 4: the lane's 8 floats are two pieces of 4, each inside the row or not at all
+      // K is a multiple of 4: a piece of 4 floats lies inside the row or not at all
+      const bool wok = c < nchunks && c * 32 + 4 * lc < K;
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
+        a0[u][h] = wok ? load_once(wl0[h] + (size_t)c * 32) : zero;
+        if (SWIGLU) a1[u][h] = wok ? load_once(wl1[h] + (size_t)c * 32) : zero;
         const bool ok = c < nchunks && k + 4 * h < K;
-        a0[u][h] = ok ? load_once(w0 + (size_t)c * 32 + 4 * h) : zero;
-        if (SWIGLU) a1[u][h] = ok ? load_once(w1 + (size_t)c * 32 + 4 * h) : zero;
         b[u][h] = (ok && xv) ? *reinterpret_cast<const float4*>(xb + (size_t)c * 32 + 4 * h) : zero;
       }
     }
 #pragma unroll
     for (int u = 0; u < kSkinnyChunks; ++u) {
+      // the lines into the wavefront's piece of shared memory, the operands out of it (one wavefront's accesses
+      // to shared memory are carried out in their order: no barrier)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const float av[4] = {a0[u][h].x, a0[u][h].y, a0[u][h].z, a0[u][h].w};
-        const float uv[4] = {a1[u][h].x, a1[u][h].y, a1[u][h].z, a1[u][h].w};
+        *reinterpret_cast<float4*>(buf0 + (8 * h + lr) * kTurnPitch + 4 * lc) = a0[u][h];
+        if (SWIGLU) *reinterpret_cast<float4*>(buf1 + (8 * h + lr) * kTurnPitch + 4 * lc) = a1[u][h];
+      }
+      float4 t0[2], t1[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        t0[h] = *reinterpret_cast<const float4*>(buf0 + r * kTurnPitch + 8 * g + 4 * h);
+        if (SWIGLU) t1[h] = *reinterpret_cast<const float4*>(buf1 + r * kTurnPitch + 8 * g + 4 * h);
+        else t1[h] = t0[h];
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const float av[4] = {t0[h].x, t0[h].y, t0[h].z, t0[h].w};
+        const float uv[4] = {t1[h].x, t1[h].y, t1[h].z, t1[h].w};
         const float bv[4] = {b[u][h].x, b[u][h].y, b[u][h].z, b[u][h].w};
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
