@@ -347,12 +347,22 @@ __global__ __launch_bounds__(kStreamWaves * 64, 2) void gemm_f32_stream_kernel(
   const float* w0 = We + (size_t)(c0 + r) * K + 8 * g;
   const float* w1 = We + (size_t)(row1 + r) * K + 8 * g;
 #define GO(NTL_) f32_stream_block<SWIGLU, NTL_>(X, w0, w1, Y, a_rows, scale, sX, tok0, live, K, Nout, c0, c1, wave_ok)
-  if (live <= 32) GO(2);
-  else if (live <= 64) GO(4);
-  else if (live <= 96) GO(6);
-  else if (live <= 128) GO(8);
-  else if (live <= 160) GO(10);
-  else GO(12);
+  // (a tile of 16 rows more or less: with a hundred rows per group the arithmetic on rows that are not there
+  // is what is left to save)
+  switch ((live + 15) >> 4) {
+    case 1: GO(1); break;
+    case 2: GO(2); break;
+    case 3: GO(3); break;
+    case 4: GO(4); break;
+    case 5: GO(5); break;
+    case 6: GO(6); break;
+    case 7: GO(7); break;
+    case 8: GO(8); break;
+    case 9: GO(9); break;
+    case 10: GO(10); break;
+    case 11: GO(11); break;
+    default: GO(12); break;
+  }
 #undef GO
 }
 
