@@ -49,14 +49,14 @@ constexpr int kSkinnyChunks = 4;  // chunks of 32 k on their way per wavefront
 // are multiplied in instructions of their own, without shared memory, was measured slower: twice the
 // instructions.)
 constexpr int kTurnPitch = 36;  // floats from row to row of a wavefront's piece of shared memory
-template <bool SWIGLU>
+template <bool SWIGLU, bool XT>
 __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
     const float* __restrict__ X, const float* __restrict__ W, float* __restrict__ Y, const int* __restrict__ offsets,
     const int* __restrict__ a_rows, const float* __restrict__ scale, int M, int Nout, int K, int num_groups,
     int slots) {
   constexpr int RT = SWIGLU ? 2 : 1;
   __shared__ float red[kSkinnyWaves][RT * 4][64];
-  __shared__ __attribute__((aligned(16))) float turn[kSkinnyWaves][RT][16 * kTurnPitch];
+  __shared__ __attribute__((aligned(16))) float turn[kSkinnyWaves][RT + (XT ? 1 : 0)][16 * kTurnPitch];  // (XT: the last holds rows of X)
   int e = blockIdx.z;
   if (slots) {
     // the blockIdx.z-th group that has rows: 64 groups per look, counted with a ballot
@@ -103,7 +103,23 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
   float* buf1 = turn[wave][RT - 1];
   const int t = tok0 + r;
   const bool xv = t < row_hi;
+  // XT (the caller expects three rows or more per group): the rows of X are read the same way (the lines of rows
+  // lr and lr + 8 of the block's 16, piece lc) and turned round in a piece of shared memory of their own: every
+  // lane's own 16 bytes of its row then cost more requests than the weights (a dense product of 8 rows took 53 us
+  // against 34 at one row; this way 40 at any number up to 16).  With one or two rows the lanes read their own
+  // pieces: the way through shared memory, and the registers and shared memory it takes from the other blocks
+  // of the compute unit, cost more than it saves there (42 against 34 us).
+  constexpr bool turn_x = XT;
   const float* xb = X + (size_t)(xv ? (a_rows != nullptr ? a_rows[t] : t) : 0) * K + 8 * g;
+  float* bufx = turn[wave][XT ? RT : 0];
+  const float* xl[2];
+  bool xlv[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int tl = tok0 + 8 * h + lr;
+    xlv[h] = tl < row_hi;
+    xl[h] = X + (size_t)(xlv[h] ? (a_rows != nullptr ? a_rows[tl] : tl) : 0) * K + 4 * lc;
+  }
   f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
   const int nchunks = (K + 31) >> 5;
   const float4 zero = {0.f, 0.f, 0.f, 0.f};
@@ -112,15 +128,18 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
 #pragma unroll
     for (int u = 0; u < kSkinnyChunks; ++u) {
       const int c = c0 + kSkinnyWaves * u;
-      const int k = c * 32 + 8 * g;
       // K is a multiple of 4: a piece of 4 floats lies inside the row or not at all
       const bool wok = c < nchunks && c * 32 + 4 * lc < K;
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         a0[u][h] = wok ? load_once(wl0[h] + (size_t)c * 32) : zero;
         if (SWIGLU) a1[u][h] = wok ? load_once(wl1[h] + (size_t)c * 32) : zero;
-        const bool ok = c < nchunks && k + 4 * h < K;
-        b[u][h] = (ok && xv) ? *reinterpret_cast<const float4*>(xb + (size_t)c * 32 + 4 * h) : zero;
+        if (turn_x) {
+          b[u][h] = (wok && xlv[h]) ? *reinterpret_cast<const float4*>(xl[h] + (size_t)c * 32) : zero;
+        } else {
+          const bool ok = c < nchunks && c * 32 + 8 * g + 4 * h < K;
+          b[u][h] = (ok && xv) ? *reinterpret_cast<const float4*>(xb + (size_t)c * 32 + 4 * h) : zero;
+        }
       }
     }
 #pragma unroll
@@ -131,10 +150,12 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
       for (int h = 0; h < 2; ++h) {
         *reinterpret_cast<float4*>(buf0 + (8 * h + lr) * kTurnPitch + 4 * lc) = a0[u][h];
         if (SWIGLU) *reinterpret_cast<float4*>(buf1 + (8 * h + lr) * kTurnPitch + 4 * lc) = a1[u][h];
+        if (turn_x) *reinterpret_cast<float4*>(bufx + (8 * h + lr) * kTurnPitch + 4 * lc) = b[u][h];
       }
-      float4 t0[2], t1[2];
+      float4 t0[2], t1[2], tx[2];
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
+        tx[h] = turn_x ? *reinterpret_cast<const float4*>(bufx + r * kTurnPitch + 8 * g + 4 * h) : b[u][h];
         t0[h] = *reinterpret_cast<const float4*>(buf0 + r * kTurnPitch + 8 * g + 4 * h);
         if (SWIGLU) t1[h] = *reinterpret_cast<const float4*>(buf1 + r * kTurnPitch + 8 * g + 4 * h);
         else t1[h] = t0[h];
@@ -143,7 +164,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
       for (int h = 0; h < 2; ++h) {
         const float av[4] = {t0[h].x, t0[h].y, t0[h].z, t0[h].w};
         const float uv[4] = {t1[h].x, t1[h].y, t1[h].z, t1[h].w};
-        const float bv[4] = {b[u][h].x, b[u][h].y, b[u][h].z, b[u][h].w};
+        const float bv[4] = {tx[h].x, tx[h].y, tx[h].z, tx[h].w};
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
           acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av[s], bv[s], acc0, 0, 0, 0);
@@ -385,10 +406,17 @@ JLE_API int jle_gemm_f32_skinny(const float* X, const float* W, float* Y, const 
   const int ytiles = (max_rows + 15) / 16;
   if (ytiles > 65535) return JLE_BAD_ARG;
   dim3 g((cols + 15) / 16, ytiles, offsets != nullptr ? (slots > 0 ? slots : G) : 1), b(kSkinnyWaves * 64);
-  if (swiglu)
-    hipLaunchKernelGGL(gemm_f32_skinny_kernel<true>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K, G, slots);
-  else
-    hipLaunchKernelGGL(gemm_f32_skinny_kernel<false>, g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K, G, slots);
+  // (rows per group that has any: at least M over the groups, or over the rows if those are fewer)
+  const int groups = offsets != nullptr ? (G < M ? G : M) : 1;
+  const bool xt = M >= 3 * groups;
+#define GO(SW_, XT_) \
+  hipLaunchKernelGGL((gemm_f32_skinny_kernel<SW_, XT_>), g, b, 0, s, X, W, Y, offsets, a_rows, scale, M, Nout, K, G, slots)
+  if (swiglu) {
+    if (xt) GO(true, true); else GO(true, false);
+  } else {
+    if (xt) GO(false, true); else GO(false, false);
+  }
+#undef GO
   JLE_LAUNCH_CHECK();
   return 0;
 }
