@@ -199,8 +199,8 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
 // ------------------------------------------------------------------------------------------ about a hundred rows
 // A prefill's rows per expert (around a hundred): every element of W should be read once, so a wavefront owns two
 // 16-row tiles of W (SWIGLU: a gate tile and its up tile) and up to 192 rows of its group, as gemm_stream.hip does
-// for bfloat16: the weights go from memory straight into the A operands (a lane's 8 consecutive floats of its row
-// feed 8 instructions, as above), the rows of X are shared by the block's wavefronts through shared memory, 32 k
+// for bfloat16: the weights go from memory into the A operands (a lane's 8 consecutive floats of its row feed 8
+// instructions; read by whole lines and turned round in the wavefront's own shared memory, as above), the rows of X are shared by the block's wavefronts through shared memory, 32 k
 // at a time (rows 144 bytes apart: the 16 lanes of an instruction's k-lane read 16 rows without meeting in a
 // bank).  A stage's weights and rows are asked for two stages ahead (a stage is thousands of cycles of arithmetic:
 // longer than a trip to memory).  K must be a multiple of 64 (whole rounds of two stages).  Groups with more than 192 rows are done in passes (each reads the weights again).
@@ -217,8 +217,9 @@ template <bool SWIGLU, int NTL>
 __device__ __forceinline__ void f32_stream_block(const float* __restrict__ X, const float* __restrict__ w0,
                                                  const float* __restrict__ w1, float* __restrict__ Y,
                                                  const int* __restrict__ a_rows, const float* __restrict__ scale,
-                                                 float (&sX)[2][kStreamRows * SPITCH], int tok0, int live, int K,
-                                                 int Nout, int c0, int c1, bool wave_ok) {
+                                                 float (&sX)[2][kStreamRows * SPITCH], float* __restrict__ turn0,
+                                                 float* __restrict__ turn1, int tok0, int live, int K, int Nout,
+                                                 int c0, int c1, bool wave_ok) {
   constexpr int THREADS = kStreamWaves * 64;
   constexpr int CHUNKS = NTL * 16 * (SBK / 4);            // 16-byte pieces of X per stage
   constexpr int CPT = (CHUNKS + THREADS - 1) / THREADS;  // per thread
@@ -249,18 +250,36 @@ __device__ __forceinline__ void f32_stream_block(const float* __restrict__ X, co
 #pragma unroll
     for (int i = 0; i < CPT; ++i) x[i] = *reinterpret_cast<const f32x4*>(X + xsrc[i] + (size_t)s * SBK);
   };
+  // w0 / w1: the first row of the wavefront's tiles.  A load instruction reads whole lines (8 lanes a row's 32 k,
+  // rows lr and lr + 8 of the tile), which are turned into the operands' order (a lane per row) through the
+  // wavefront's own pieces of shared memory turn0 / turn1, as in the kernel for few rows.
+  const int lr = lane >> 3, lc = lane & 7;
+  const float* wl0 = w0 + (size_t)lr * K + 4 * lc;
+  const float* wl1 = w1 + (size_t)lr * K + 4 * lc;
   auto ask_weights = [&](f32x4 (&w)[2][2], int s) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      w[0][h] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(w0 + (size_t)s * SBK + 4 * h));
-      w[1][h] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(w1 + (size_t)s * SBK + 4 * h));
+      w[0][h] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wl0 + (size_t)(8 * h) * K + (size_t)s * SBK));
+      w[1][h] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wl1 + (size_t)(8 * h) * K + (size_t)s * SBK));
     }
   };
   auto put = [&](const f32x4 (&x)[CPT], float* buf) {
 #pragma unroll
     for (int i = 0; i < CPT; ++i) *reinterpret_cast<f32x4*>(buf + xdst[i]) = x[i];
   };
-  auto work = [&](const f32x4 (&w)[2][2], const float* buf) {
+  auto work = [&](const f32x4 (&wl)[2][2], const float* buf) {
+    // (one wavefront's accesses to shared memory are carried out in their order: no barrier)
+    f32x4 w[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      *reinterpret_cast<f32x4*>(turn0 + (8 * h + lr) * kTurnPitch + 4 * lc) = wl[0][h];
+      *reinterpret_cast<f32x4*>(turn1 + (8 * h + lr) * kTurnPitch + 4 * lc) = wl[1][h];
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      w[0][h] = *reinterpret_cast<const f32x4*>(turn0 + r * kTurnPitch + 8 * g + 4 * h);
+      w[1][h] = *reinterpret_cast<const f32x4*>(turn1 + r * kTurnPitch + 8 * g + 4 * h);
+    }
     // (the next tile's rows are read while this tile's 16 instructions run, and no further ahead: left to itself
     // the compiler reads all tiles' rows first and runs out of registers)
     f32x4 blo = *reinterpret_cast<const f32x4*>(buf + b_off);
@@ -334,6 +353,7 @@ __global__ __launch_bounds__(kStreamWaves * 64, 2) void gemm_f32_stream_kernel(
     const float* __restrict__ X, const float* __restrict__ W, float* __restrict__ Y, const int* __restrict__ offsets,
     const int* __restrict__ a_rows, const float* __restrict__ scale, int M, int Nout, int K, int nblk, int passes) {
   __shared__ __attribute__((aligned(16))) float sX[2][kStreamRows * SPITCH];
+  __shared__ __attribute__((aligned(16))) float turn[kStreamWaves][2][16 * kTurnPitch];
   const int item = blockIdx.x;
   const int nb = item % nblk, pass = (item / nblk) % passes, e = item / (nblk * passes);
   int row_lo = 0, row_hi = M;
@@ -365,9 +385,11 @@ __global__ __launch_bounds__(kStreamWaves * 64, 2) void gemm_f32_stream_kernel(
     c1 = min(c0 + 16, (ntile - 1) * 16);
     row1 = c1;
   }
-  const float* w0 = We + (size_t)(c0 + r) * K + 8 * g;
-  const float* w1 = We + (size_t)(row1 + r) * K + 8 * g;
-#define GO(NTL_) f32_stream_block<SWIGLU, NTL_>(X, w0, w1, Y, a_rows, scale, sX, tok0, live, K, Nout, c0, c1, wave_ok)
+  const float* w0 = We + (size_t)c0 * K;
+  const float* w1 = We + (size_t)row1 * K;
+#define GO(NTL_)                                                                                                     \
+  f32_stream_block<SWIGLU, NTL_>(X, w0, w1, Y, a_rows, scale, sX, turn[wave][0], turn[wave][1], tok0, live, K, Nout, \
+                                 c0, c1, wave_ok)
   // (a tile of 16 rows more or less: with a hundred rows per group the arithmetic on rows that are not there
   // is what is left to save)
   switch ((live + 15) >> 4) {
