@@ -200,10 +200,12 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_f32_skinny_kernel(
 // A prefill's rows per expert (around a hundred): every element of W should be read once, so a wavefront owns two
 // 16-row tiles of W (SWIGLU: a gate tile and its up tile) and up to 192 rows of its group, as gemm_stream.hip does
 // for bfloat16: the weights go from memory into the A operands (a lane's 8 consecutive floats of its row feed 8
-// instructions; read by whole lines and turned round in the wavefront's own shared memory, as above), the rows of X are shared by the block's wavefronts through shared memory, 32 k
-// at a time (rows 144 bytes apart: the 16 lanes of an instruction's k-lane read 16 rows without meeting in a
-// bank).  A stage's weights and rows are asked for two stages ahead (a stage is thousands of cycles of arithmetic:
-// longer than a trip to memory).  K must be a multiple of 64 (whole rounds of two stages).  Groups with more than 192 rows are done in passes (each reads the weights again).
+// instructions; read by whole lines and turned round in the wavefront's own shared memory, as above), the rows
+// of X are shared by the block's wavefronts through shared memory, 32 k at a time (rows 144 bytes apart: the 16
+// lanes of an instruction's k-lane read 16 rows without meeting in a bank).  A stage's weights and rows are asked
+// for two stages ahead (a stage is thousands of cycles of arithmetic: longer than a trip to memory).  K must be
+// a multiple of 64 (whole rounds of two stages).  Groups with more than 192 rows are done in passes (each reads
+// the weights again).
 // The arithmetic is the limit here (each instruction is 2,048 operations in 32 cycles of a SIMD), not the stream.
 //
 // Order of the sums: over the stages in ascending order, within a stage as in the kernel above; it depends on K
