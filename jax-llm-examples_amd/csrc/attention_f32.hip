@@ -106,18 +106,34 @@ __global__ __launch_bounds__(256) void attention_f32_tiles_kernel(
     key_lo += sp * keys_per_split;
     key_hi = min(pos_last, key_lo + keys_per_split - 1);
   }
-  for (int key0 = key_lo; key0 <= key_hi; key0 += 16) {
+  // A step's keys and values are asked for while the step before it is worked on (two sets of registers, taken
+  // in turn): a step is a few dozen dependent instructions, a trip to memory takes several times as long.
+  // fetch: this lane's row of key key0 + c16 (A operand of the scores) and 4 consecutive keys of its head elements
+  // (A operand of the values); the step's page (-1: none), the same in all lanes.
+  auto fetch = [&](int key0, float4 (&ka)[DT], float4 (&va)[DT], int& page_step) {
+    const int kk = key0 + c16;
+    const bool key_there = kk >= lo && kk <= pos_last;
+    const int page_a = key_there ? table[kk / ps] : -1;
+    const float* krow = kv + (size_t)max(page_a, 0) * page_stride + head_off + (size_t)(kk % ps) * dh + 4 * g;
+    page_step = table[key0 / ps];  // (a step lies in one page)
+    const float* vbase = kv + (size_t)max(page_step, 0) * page_stride + head_off + v_off + (key0 % ps) + 4 * g;
+#pragma unroll
+    for (int c = 0; c < DT; ++c) {
+      ka[c] = float4{0.f, 0.f, 0.f, 0.f};
+      va[c] = float4{0.f, 0.f, 0.f, 0.f};
+      if (c < dt) {
+        if (page_a >= 0) ka[c] = *reinterpret_cast<const float4*>(krow + 16 * c);
+        if (page_step >= 0) va[c] = *reinterpret_cast<const float4*>(vbase + (size_t)(16 * c + c16) * ps);
+      }
+    }
+  };
+  auto work = [&](int key0, const float4 (&ka)[DT], const float4 (&va)[DT], int page_step) {
     // ---- scores of the step's 16 keys for the tile's queries
-    const int ka = key0 + c16;  // the key whose row this lane brings (A operand)
-    const bool key_there = ka >= lo && ka <= pos_last;
-    const int page_a = key_there ? table[ka / ps] : -1;
-    const float* krow = kv + (size_t)max(page_a, 0) * page_stride + head_off + (size_t)(ka % ps) * dh + 4 * g;
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < DT; ++c) {
       if (c < dt) {
-        float4 a = {0.f, 0.f, 0.f, 0.f};
-        if (page_a >= 0) a = *reinterpret_cast<const float4*>(krow + 16 * c);
+        const float4 a = ka[c];
         s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, qreg[c].x, s, 0, 0, 0);
         s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, qreg[c].y, s, 0, 0, 0);
         s = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, qreg[c].z, s, 0, 0, 0);
@@ -125,7 +141,6 @@ __global__ __launch_bounds__(256) void attention_f32_tiles_kernel(
       }
     }
     // s[v]: key key0 + 4 g + v, query c16.  A key a query may read whose page is not there is an error.
-    const int page_step = table[key0 / ps];  // (a step lies in one page)
     float p[4];
     float mx = -INFINITY;
 #pragma unroll
@@ -152,9 +167,8 @@ __global__ __launch_bounds__(256) void attention_f32_tiles_kernel(
     for (int t = 0; t < DT; ++t)
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[t][v] *= corr;
-    // ---- values: this lane brings 4 consecutive keys of head element 16 t + c16
-    if (page_step < 0) continue;  // (the same for the whole wavefront)
-    const float* vbase = kv + (size_t)page_step * page_stride + head_off + v_off + (key0 % ps) + 4 * g;
+    // ---- values: this lane brought 4 consecutive keys of head element 16 t + c16
+    if (page_step < 0) return;  // (the same for the whole wavefront)
     // keys outside [lo, pos_last] may hold anything (slots never written, or written by an earlier holder of the
     // page): they count with probability 0, and 0 times a stray NaN would still be NaN
     bool kv_ok[4];
@@ -166,12 +180,33 @@ __global__ __launch_bounds__(256) void attention_f32_tiles_kernel(
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
       if (t < dt) {
-        const float4 a = *reinterpret_cast<const float4*>(vbase + (size_t)(16 * t + c16) * ps);
+        const float4 a = va[t];
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv_ok[0] ? a.x : 0.f, p[0], acc[t], 0, 0, 0);
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv_ok[1] ? a.y : 0.f, p[1], acc[t], 0, 0, 0);
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv_ok[2] ? a.z : 0.f, p[2], acc[t], 0, 0, 0);
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv_ok[3] ? a.w : 0.f, p[3], acc[t], 0, 0, 0);
       }
+    }
+  };
+  if constexpr (HEADS) {
+    float4 ka0[DT], va0[DT], ka1[DT], va1[DT];
+    int page0 = -1, page1 = -1;
+    if (key_lo <= key_hi) fetch(key_lo, ka0, va0, page0);
+    for (int key0 = key_lo; key0 <= key_hi; key0 += 32) {
+      if (key0 + 16 <= key_hi) fetch(key0 + 16, ka1, va1, page1);
+      work(key0, ka0, va0, page0);
+      if (key0 + 16 > key_hi) break;
+      if (key0 + 32 <= key_hi) fetch(key0 + 32, ka0, va0, page0);
+      work(key0 + 16, ka1, va1, page1);
+    }
+  } else {
+    // (portions of prompts: many wavefronts per SIMD hide the trips to memory; a second set of registers would
+    // halve their number: measured 1,178 against 1,127 us a layer at 2,048 tokens)
+    for (int key0 = key_lo; key0 <= key_hi; key0 += 16) {
+      float4 ka[DT], va[DT];
+      int page = -1;
+      fetch(key0, ka, va, page);
+      work(key0, ka, va, page);
     }
   }
   bad = __any(bad);
