@@ -185,25 +185,43 @@ __global__ __launch_bounds__(256) void paged_attention_generic_merge_kernel(cons
   const int nh = blockIdx.x * 4 + wave_index();
   if (nh >= NH) return;
   const float* ml = ws_ml + (size_t)nh * splits * 2;
+  // the ranges' maxima: a lane per range (64 at a time), then across the lanes; every trip to memory of a pass is
+  // under way at once
   float mx = -INFINITY;
   bool bad = false;
-  for (int sp = 0; sp < splits; ++sp) {
-    const float ms = ml[sp * 2];
+  for (int s0 = 0; s0 < splits; s0 += 64) {
+    const float ms = s0 + lane < splits ? ml[(s0 + lane) * 2] : -INFINITY;
     bad |= ms != ms;  // a missing page
     mx = fmaxf(mx, ms);
   }
+  bad = __any(bad);
+  mx = wave_max(mx);  // (the same value whatever the order: a maximum)
+  // the sums in the ranges' order, as ever; eight ranges' rows are asked for before the first is added
   float l = 0.f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int sp = 0; sp < splits; ++sp) {
-    const float ms = ml[sp * 2];
-    if (ms == -INFINITY || ms != ms) continue;  // a range without keys
-    const float wgt = expf(ms - mx);
-    l += ml[sp * 2 + 1] * wgt;
-    const float* o = ws_o + ((size_t)nh * splits + sp) * dh;
+  constexpr int U = 8;
+  for (int s0 = 0; s0 < splits; s0 += U) {
+    float ms[U], ls[U], o[U][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int d = lane + 64 * i;
-      if (d < dh) acc[i] += o[d] * wgt;
+    for (int u = 0; u < U; ++u) {
+      const int sp = min(s0 + u, splits - 1);  // (past the last: loaded again, not used)
+      ms[u] = ml[sp * 2];
+      ls[u] = ml[sp * 2 + 1];
+      const float* row = ws_o + ((size_t)nh * splits + sp) * dh;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = lane + 64 * i;
+        o[u][i] = d < dh ? row[d] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (s0 + u >= splits) break;
+      if (ms[u] == -INFINITY || ms[u] != ms[u]) continue;  // a range without keys
+      const float wgt = expf(ms[u] - mx);
+      l += ls[u] * wgt;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] += o[u][i] * wgt;
     }
   }
   const float inv = bad ? __builtin_nanf("") : 1.0f / l;
